@@ -1,0 +1,142 @@
+"""Parity of the whole-model path (wgpt_prefill / wgpt_decode / wgpt_decode_greedy,
+called through the C ABI) against the CPU oracle's GPT.run restatement."""
+import numpy as np
+import pytest
+
+from oracle import ref
+from webgpt_amd import WgptError, _lib, synth
+from webgpt_amd.model import GPT
+
+from helpers import close, make_model, oracle_weights, small_cfg, worst
+
+pytestmark = pytest.mark.gpu
+
+
+def load(cfg, seed, flags=0, random_ln=True):
+    tensors = make_model(cfg, seed, random_ln=random_ln)
+    gpt = GPT(None, "char", tensors=tensors, params=synth.model_params(cfg), flags=flags)
+    gpt.initialize()
+    return gpt, tensors
+
+
+def greedy_ok(got_logits, want_logits):
+    """Greedy ids must agree unless the oracle's top-2 gap is inside the tolerance."""
+    g, w = int(np.argmax(got_logits)), int(np.argmax(want_logits))
+    if g == w:
+        return True
+    top2 = np.sort(want_logits)[-2:]
+    return abs(float(top2[1] - top2[0])) <= 1e-5 + 1e-4 * abs(float(top2[1]))
+
+
+@pytest.mark.parametrize("cfg,T", [(small_cfg(), 1), (small_cfg(), 9), (small_cfg(n_layer=3, n_head=4, n_embd=64, n_ctx=40, vocab_size=97), 40),
+                                   (dict(synth.CONFIGS["toy"]), 64)])
+def test_prefill_taps_and_logits(device, cfg, T):
+    gpt, tensors = load(cfg, seed=11, flags=_lib.FLAG_TAPS)
+    tokens = synth.tokens(5, "prompt", T, cfg["vocab_size"])
+    want_logits, want_taps, want_kv = ref.forward(synth.model_params(cfg), oracle_weights(tensors, cfg), tokens,
+                                                  want_taps=True, want_kv=True)
+    logits = gpt.prefill(tokens)
+    for i, name in enumerate(ref.tap_names(cfg["n_layer"])):
+        got = gpt.tap(name, T)
+        assert close(got, want_taps[i]), (name, worst(got, want_taps[i]))
+    for i in range(cfg["n_layer"]):
+        assert close(gpt.tap(f"kv{i}_k"), want_kv[i, 0]) and close(gpt.tap(f"kv{i}_v"), want_kv[i, 1])
+    assert close(logits, want_logits), worst(logits, want_logits)
+    assert greedy_ok(logits, want_logits)
+    gpt.unloadBuffers()
+
+
+def test_decode_equals_last_row_of_full_forward(device):
+    # decode(t) with the KV cache must equal the reference's full-window recompute of tokens [0..t]
+    cfg = dict(synth.CONFIGS["toy"])
+    gpt, tensors = load(cfg, seed=7)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(3, "prompt", 40, cfg["vocab_size"])
+    logits = gpt.run(tokens[:8])
+    assert close(logits, ref.forward(p, w, tokens[:8]))
+    for t in range(8, 40):
+        logits = gpt.run(tokens[: t + 1])          # extends the window by one: served from the cache
+        if t in (8, 9, 17, 31, 39):
+            want = ref.forward(p, w, tokens[: t + 1])
+            assert close(logits, want), (t, worst(logits, want))
+            assert greedy_ok(logits, want)
+    # a window that is not an extension recomputes from scratch
+    other = synth.tokens(4, "prompt", 5, cfg["vocab_size"])
+    assert close(gpt.run(other), ref.forward(p, w, other))
+    gpt.unloadBuffers()
+
+
+def test_greedy_generation_matches_oracle(device):
+    cfg = dict(synth.CONFIGS["toy"])
+    gpt, tensors = load(cfg, seed=1, random_ln=False)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    prompt = [int(t) for t in synth.make_prompt(cfg, 1, 16)]
+    # host loop (GPT.generate with top_k = 1)
+    host_ids = list(gpt.generate(prompt, 12, 1, 1.0))
+    # oracle loop: full-window recompute per token, as the reference does
+    hist = list(prompt)
+    for i in range(12):
+        lg = ref.forward(p, w, np.array(hist, np.int32))
+        nxt = int(np.argmax(lg))
+        if nxt != host_ids[i]:
+            assert greedy_ok(gpt.run(hist), lg)
+            break
+        hist.append(nxt)
+    # device loop: prefill, then all steps on the device
+    lg = gpt.prefill(prompt)
+    first = int(np.argmax(lg))
+    dev_ids, last_logits = gpt.decode_greedy(first, 11, want_logits=True)
+    assert [first] + [int(t) for t in dev_ids[:-1]] == host_ids[:12]
+    gpt.unloadBuffers()
+
+
+def test_context_limit_and_errors(device):
+    cfg = small_cfg(n_ctx=12)
+    gpt, tensors = load(cfg, seed=2)
+    tokens = synth.tokens(3, "prompt", 12, cfg["vocab_size"])
+    gpt.prefill(tokens[:11])
+    gpt.decode(int(tokens[11]))
+    with pytest.raises(WgptError, match="context"):
+        gpt.decode(1)
+    with pytest.raises(WgptError, match="outside"):
+        gpt.prefill([cfg["vocab_size"]])
+    with pytest.raises(WgptError, match="exceeds"):
+        gpt.prefill(np.zeros(13, np.int32))
+    # sliding the window (model.js:69): recompute on the last n_ctx tokens, positions restart at 0
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    hist = list(tokens) + [5, 6]
+    got = gpt.run(hist[-12:])
+    assert close(got, ref.forward(p, w, np.array(hist[-12:], np.int32)))
+    gpt.unloadBuffers()
+
+
+def test_int8_model(device):
+    cfg = small_cfg(n_layer=2, n_head=2, n_embd=64, n_ctx=24, vocab_size=50, dtype="int8")
+    gpt, tensors = load(cfg, seed=13)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(3, "prompt", 12, cfg["vocab_size"])
+    for T in (3, 9):      # GEMV path (<= 4 rows) and the dequantise + GEMM path
+        got = gpt.prefill(tokens[:T])
+        want = ref.forward(p, w, tokens[:T])
+        assert close(got, want), worst(got, want)
+    got = gpt.run(tokens[:10])
+    want = ref.forward(p, w, tokens[:10])
+    assert close(got, want), worst(got, want)
+    gpt.unloadBuffers()
+
+
+def test_gpt2_117m_shape_prefill_and_decode(device):
+    cfg = dict(synth.CONFIGS["gpt2-117m"])
+    gpt, tensors = load(cfg, seed=1, random_ln=False)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.make_prompt(cfg, 1, 24)
+    got = gpt.prefill(tokens[:20])
+    want = ref.forward(p, w, tokens[:20])
+    assert close(got, want), worst(got, want)
+    for t in range(20, 24):
+        got = gpt.decode(int(tokens[t]))
+    want = ref.forward(p, w, tokens[:24])
+    assert close(got, want), worst(got, want)
+    assert greedy_ok(got, want)
+    assert gpt.decode_bytes(0) == 4 * (12 * (12 * 768 * 768 + 13 * 768) + 50257 * 768 + 2 * 768)
+    gpt.unloadBuffers()

@@ -1,0 +1,55 @@
+// Launchers of the per-block HIP kernels. All take raw device pointers that the
+// caller has already validated against the shapes given; all enqueue on `s`.
+#ifndef WGPT_KERNELS_H
+#define WGPT_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace wgpt {
+
+enum Epilogue { EPI_NONE = 0, EPI_GELU = 1, EPI_RESIDUAL = 2 };
+
+// Rows handled per pass of the GEMV path; a matmul with M <= this is a GEMV.
+constexpr int GEMV_MAX_ROWS = 4;
+constexpr int GEMV_KCHUNK = 64;
+
+// Floats of workspace the GEMV path needs for C[M,N] = A[M,K] . W[K,N].
+size_t gemv_workspace_floats(int M, int N, int K);
+
+// C[M,ldc] = epi(A[M,K] . W[K,N] (row stride ldw) + bias) for M <= GEMV_MAX_ROWS.
+// bias may be null. resid (EPI_RESIDUAL) has row stride ldc and may alias C.
+hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
+                          float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
+
+// Same contraction for any M through the tiled GEMM kernels.
+hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
+                       float* C, int ldc, int epi, const float* resid, hipStream_t s);
+
+// int8 weight-only variants: Wq is [K, ldwq] words holding 4 columns each.
+hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,
+                             const float* scale, const float* bias, float* C, int ldc, int epi, const float* resid,
+                             float* workspace, hipStream_t s);
+hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const float* scale, float* W, int ldw, hipStream_t s);
+
+hipError_t launch_residual(size_t n4, const float* a, const float* b, float* out, hipStream_t s);
+hipError_t launch_gelu(size_t n4, const float* x, float* out, hipStream_t s);
+hipError_t launch_layernorm(int M, int N, const float* x, int ldx, const float* gamma, const float* beta, float* out, int ldo,
+                            hipStream_t s);
+hipError_t launch_softmax(int M, int N, const float* x, float* out, hipStream_t s);
+// out[i,:] = wte[idx[i],:] + wpe[pos0+i,:]; idx on the device.
+hipError_t launch_embed(const int32_t* idx, int T, int d, int pos0, const float* wte, const float* wpe, float* out, hipStream_t s);
+// logits[v] = x . wte[v,:]
+hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, float* logits, hipStream_t s);
+// Causal attention of Tq query rows (absolute positions pos0..pos0+Tq-1) against
+// keys/values 0..pos of a [ctx, d]-shaped cache. q row i is at q + i*ldq + h*hs.
+hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
+                            const float* Vc, int ldkv, float* out, int ldo, hipStream_t s);
+// Copies rows of src (row stride lds, `cols` floats wide) to dst (row stride ldd).
+hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float* dst, int ldd, hipStream_t s);
+// tok[0] = argmax(logits[0..V)) with the lowest index on ties; also stored to out[slot].
+hipError_t launch_argmax(int V, const float* logits, int32_t* tok, int32_t* out, int slot, hipStream_t s);
+
+}  // namespace wgpt
+
+#endif

@@ -1,0 +1,577 @@
+// Per-block HIP kernels for gfx950 (wave64). One kernel family per instruction
+// block of the reference (instructions.js); the arithmetic each one reproduces is
+// cited at the kernel. Summation orders differ from the WGSL (lanes split the
+// reduction and combine by wave shuffles), which stays inside the fp32 tolerance.
+#include "kernels.h"
+
+namespace wgpt {
+
+namespace {
+
+constexpr int WG = 256;     // threads per workgroup for every kernel here
+constexpr int NWAVE = WG / 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  return v;
+}
+
+// Sum over a 256-thread workgroup; `sh` holds NWAVE floats. Every thread gets the result.
+__device__ __forceinline__ float block_sum(float v, float* sh) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+  __syncthreads();
+  return v;
+}
+
+__device__ __forceinline__ float block_max(float v, float* sh) {
+  v = wave_max(v);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  __syncthreads();
+  return v;
+}
+
+// GELU of the reference, instructions.js:718-727: tanh form, exact 0 below -10,
+// identity above 10; x^3 as x*x*x.
+__device__ __forceinline__ float gelu_ref(float x) {
+  const float x3 = x * x * x;
+  const float cdf = 0.5f * (1.0f + tanhf(0.7978845608f * (x + 0.044715f * x3)));
+  float r = x * cdf;
+  r = x < -10.0f ? 0.0f : r;
+  r = x > 10.0f ? x : r;
+  return r;
+}
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+
+__device__ __forceinline__ void fma4(float4& acc, float a, const float4& w) {
+  acc.x += a * w.x;
+  acc.y += a * w.y;
+  acc.z += a * w.z;
+  acc.w += a * w.w;
+}
+
+// unpackInt8x4, other/int8-gemm.js:126-132: sign-extend each byte, then
+// f32(b) / 127.0 * scale with a rounding after the divide and after the multiply.
+__device__ __forceinline__ float4 unpack_i8x4(int32_t word, const float4& sc) {
+  const int b0 = (word << 24) >> 24;
+  const int b1 = (word << 16) >> 24;
+  const int b2 = (word << 8) >> 24;
+  const int b3 = word >> 24;
+  float4 r;
+  r.x = __fdiv_rn((float)b0, 127.0f) * sc.x;
+  r.y = __fdiv_rn((float)b1, 127.0f) * sc.y;
+  r.z = __fdiv_rn((float)b2, 127.0f) * sc.z;
+  r.w = __fdiv_rn((float)b3, 127.0f) * sc.w;
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// FastMatMulBlock for M <= 4 (batch-1 decode): C = A . W + bias,
+// instructions.js:248-314. W is [K,N] row-major as the reference keeps it.
+// Stage 1: a workgroup owns a 64-column x 64-row tile of W; 16 lanes read one
+// 256-byte row segment as float4s, the 16 lane groups take rows k0+ty, +16, ...
+// and combine through LDS. Stage 2 sums the K/64 partials in ascending order,
+// adds the bias last (as the shader does) and applies the epilogue.
+// ---------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(WG) void gemv_kn_partial(int N, int K, const float* __restrict__ A, int lda,
+                                                       const float* __restrict__ W, int ldw, float* __restrict__ part) {
+  __shared__ float4 red[R][16][16];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int n0 = blockIdx.x * 64 + tx * 4;
+  const int k0 = blockIdx.y * GEMV_KCHUNK;
+  float4 acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (n0 < N) {
+#pragma unroll
+    for (int i = 0; i < GEMV_KCHUNK / 16; ++i) {
+      const int k = k0 + ty + 16 * i;
+      if (k < K) {
+        const float4 w = ld4(W + (size_t)k * ldw + n0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) fma4(acc[r], A[(size_t)r * lda + k], w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) red[r][ty][tx] = acc[r];
+  __syncthreads();
+  if (ty < R && n0 < N) {
+    float4 s = red[ty][0][tx];
+#pragma unroll
+    for (int j = 1; j < 16; ++j) {
+      const float4 v = red[ty][j][tx];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    st4(part + ((size_t)blockIdx.y * R + ty) * N + n0, s);
+  }
+}
+
+__global__ __launch_bounds__(WG) void gemv_reduce(int M, int N, int S, const float* __restrict__ part,
+                                                   const float* __restrict__ bias, float* C, int ldc, int epi,
+                                                   const float* resid) {
+  const int n4 = N >> 2;
+  const int idx = blockIdx.x * WG + threadIdx.x;
+  if (idx >= M * n4) return;
+  const int r = idx / n4, n0 = (idx - r * n4) * 4;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int sp = 0; sp < S; ++sp) {
+    const float4 v = ld4(part + ((size_t)sp * M + r) * N + n0);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (bias) {
+    const float4 b = ld4(bias + n0);
+    s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+  }
+  if (epi == EPI_GELU) {
+    s.x = gelu_ref(s.x); s.y = gelu_ref(s.y); s.z = gelu_ref(s.z); s.w = gelu_ref(s.w);
+  } else if (epi == EPI_RESIDUAL) {
+    const float4 q = ld4(resid + (size_t)r * ldc + n0);
+    s.x += q.x; s.y += q.y; s.z += q.z; s.w += q.w;
+  }
+  st4(C + (size_t)r * ldc + n0, s);
+}
+
+// int8 weight-only stage 1 (other/int8-gemm.js:156-210 at M <= 4): a wave reads
+// 64 consecutive words (256 columns) of one row; 4 waves take rows k0+ty, +4, ...
+template <int R>
+__global__ __launch_bounds__(WG) void gemv_kn_i8_partial(int N, int K, const float* __restrict__ A, int lda,
+                                                          const int32_t* __restrict__ Wq, int ldwq,
+                                                          const float* __restrict__ scale, float* __restrict__ part) {
+  __shared__ float4 red[R][NWAVE][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 256 + tx * 4;
+  const int k0 = blockIdx.y * GEMV_KCHUNK;
+  float4 acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (n0 < N) {
+    const float4 sc = ld4(scale + n0);
+#pragma unroll 4
+    for (int i = 0; i < GEMV_KCHUNK / NWAVE; ++i) {
+      const int k = k0 + ty + NWAVE * i;
+      if (k < K) {
+        const float4 w = unpack_i8x4(Wq[(size_t)k * ldwq + (n0 >> 2)], sc);
+#pragma unroll
+        for (int r = 0; r < R; ++r) fma4(acc[r], A[(size_t)r * lda + k], w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) red[r][ty][tx] = acc[r];
+  __syncthreads();
+  if (ty < R && n0 < N) {
+    float4 s = red[ty][0][tx];
+#pragma unroll
+    for (int j = 1; j < NWAVE; ++j) {
+      const float4 v = red[ty][j][tx];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    st4(part + ((size_t)blockIdx.y * R + ty) * N + n0, s);
+  }
+}
+
+__global__ __launch_bounds__(WG) void dequant_i8_kernel(int K, int N, const int32_t* __restrict__ Wq, int ldwq,
+                                                         const float* __restrict__ scale, float* __restrict__ W, int ldw) {
+  const int n4 = N >> 2;
+  const size_t idx = (size_t)blockIdx.x * WG + threadIdx.x;
+  if (idx >= (size_t)K * n4) return;
+  const int k = (int)(idx / n4), w = (int)(idx - (size_t)k * n4);
+  st4(W + (size_t)k * ldw + 4 * w, unpack_i8x4(Wq[(size_t)k * ldwq + w], ld4(scale + 4 * w)));
+}
+
+// ---------------------------------------------------------------------------
+// FastMatMulBlock for any M (prefill): 64x64 output tile per workgroup, 4x4 per
+// thread, K in steps of 16 through LDS. Same contraction and bias-last order of
+// operations per element as instructions.js:248-314 up to fp32 reassociation.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(WG) void gemm_tile64(int M, int N, int K, const float* __restrict__ A, int lda,
+                                                   const float* __restrict__ W, int ldw, const float* __restrict__ bias,
+                                                   float* C, int ldc, int epi, const float* resid) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Bs[16][64];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tm = tid >> 4, tn = tid & 15;
+  const int arow = tid >> 2, akq = (tid & 3) * 4;
+  const int brow = tid >> 4, bnq = (tid & 15) * 4;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    float4 av = make_float4(0.f, 0.f, 0.f, 0.f), bv = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (m0 + arow < M && k0 + akq < K) av = ld4(A + (size_t)(m0 + arow) * lda + k0 + akq);
+    if (k0 + brow < K && n0 + bnq < N) bv = ld4(W + (size_t)(k0 + brow) * ldw + n0 + bnq);
+    As[akq + 0][arow] = av.x;
+    As[akq + 1][arow] = av.y;
+    As[akq + 2][arow] = av.z;
+    As[akq + 3][arow] = av.w;
+    st4(&Bs[brow][bnq], bv);
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      const float4 a = ld4(&As[kk][tm * 4]);
+      const float4 b = ld4(&Bs[kk][tn * 4]);
+      const float aa[4] = {a.x, a.y, a.z, a.w};
+      const float bb[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += aa[i] * bb[j];
+    }
+    __syncthreads();
+  }
+  const int n = n0 + tn * 4;
+  if (n >= N) return;
+  float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) b = ld4(bias + n);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + tm * 4 + i;
+    if (m >= M) break;
+    float4 v = make_float4(acc[i][0] + b.x, acc[i][1] + b.y, acc[i][2] + b.z, acc[i][3] + b.w);
+    if (epi == EPI_GELU) {
+      v.x = gelu_ref(v.x); v.y = gelu_ref(v.y); v.z = gelu_ref(v.z); v.w = gelu_ref(v.w);
+    } else if (epi == EPI_RESIDUAL) {
+      const float4 q = ld4(resid + (size_t)m * ldc + n);
+      v.x += q.x; v.y += q.y; v.z += q.z; v.w += q.w;
+    }
+    st4(C + (size_t)m * ldc + n, v);
+  }
+}
+
+// ResidualBlock, instructions.js:381-382
+__global__ __launch_bounds__(WG) void residual_kernel(size_t n4, const float* a, const float* b, float* out) {
+  const size_t i = (size_t)blockIdx.x * WG + threadIdx.x;
+  if (i >= n4) return;
+  const float4 x = ld4(a + 4 * i), y = ld4(b + 4 * i);
+  st4(out + 4 * i, make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w));
+}
+
+// GeluBlock, instructions.js:718-746
+__global__ __launch_bounds__(WG) void gelu_kernel(size_t n4, const float* x, float* out) {
+  const size_t i = (size_t)blockIdx.x * WG + threadIdx.x;
+  if (i >= n4) return;
+  const float4 v = ld4(x + 4 * i);
+  st4(out + 4 * i, make_float4(gelu_ref(v.x), gelu_ref(v.y), gelu_ref(v.z), gelu_ref(v.w)));
+}
+
+// LayerNormBlock: stats pass + norm pass of instructions.js:451-550 in one kernel,
+// one workgroup per row. mean = sum/N; var = sum((x-mean)^2)/N; stdev = sqrt(var + 1e-5);
+// out = gamma * ((x - mean) / stdev) + beta with a true division.
+__global__ __launch_bounds__(WG) void layernorm_kernel(int N, const float* __restrict__ x, int ldx,
+                                                        const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                        float* __restrict__ out, int ldo) {
+  __shared__ float sh[NWAVE];
+  const float* xr = x + (size_t)blockIdx.x * ldx;
+  float* orow = out + (size_t)blockIdx.x * ldo;
+  const int n4 = N >> 2;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n4; i += WG) {
+    const float4 v = ld4(xr + 4 * i);
+    s += (v.x + v.y) + (v.z + v.w);
+  }
+  const float mean = block_sum(s, sh) / (float)N;
+  float q = 0.f;
+  for (int i = threadIdx.x; i < n4; i += WG) {
+    const float4 v = ld4(xr + 4 * i);
+    const float a = v.x - mean, b = v.y - mean, c = v.z - mean, d = v.w - mean;
+    q += (a * a + b * b) + (c * c + d * d);
+  }
+  const float var = block_sum(q, sh) / (float)N;
+  const float stdev = sqrtf(var + 1e-5f);
+  for (int i = threadIdx.x; i < n4; i += WG) {
+    const float4 v = ld4(xr + 4 * i), g = ld4(gamma + 4 * i), b = ld4(beta + 4 * i);
+    float4 o;
+    o.x = g.x * ((v.x - mean) / stdev) + b.x;
+    o.y = g.y * ((v.y - mean) / stdev) + b.y;
+    o.z = g.z * ((v.z - mean) / stdev) + b.z;
+    o.w = g.w * ((v.w - mean) / stdev) + b.w;
+    st4(orow + 4 * i, o);
+  }
+}
+
+// SoftmaxBlock, instructions.js:618-663: max from -3.402823e38, sum of exp(x - max),
+// out = exp(x - max) / sum with the exponential recomputed and a true division.
+__global__ __launch_bounds__(WG) void softmax_kernel(int N, const float* __restrict__ x, float* __restrict__ out) {
+  __shared__ float sh[NWAVE];
+  const float* xr = x + (size_t)blockIdx.x * N;
+  float* orow = out + (size_t)blockIdx.x * N;
+  float m = -3.402823e+38f;
+  for (int i = threadIdx.x; i < N; i += WG) m = fmaxf(m, xr[i]);
+  m = block_max(m, sh);
+  float s = 0.f;
+  for (int i = threadIdx.x; i < N; i += WG) s += expf(xr[i] - m);
+  s = block_sum(s, sh);
+  for (int i = threadIdx.x; i < N; i += WG) orow[i] = expf(xr[i] - m) / s;
+}
+
+// EmbedBlock, instructions.js:795-821: gather + positional add in one pass.
+__global__ __launch_bounds__(WG) void embed_kernel(const int32_t* __restrict__ idx, int d, int pos0,
+                                                    const float* __restrict__ wte, const float* __restrict__ wpe,
+                                                    float* __restrict__ out) {
+  const int i = blockIdx.x;
+  const size_t tok = (size_t)idx[i];
+  const float* e = wte + tok * d;
+  const float* p = wpe + (size_t)(pos0 + i) * d;
+  for (int c = threadIdx.x; c < (d >> 2); c += WG) {
+    const float4 a = ld4(e + 4 * c), b = ld4(p + 4 * c);
+    st4(out + (size_t)i * d + 4 * c, make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w));
+  }
+}
+
+// DeEmbedBlock, instructions.js:916-943, on the un-chunked, un-transposed wte[V,d]:
+// row-major wte already has the contraction index contiguous, so a wave streams
+// whole rows with 128-bit loads and reduces by shuffles. 4 rows per wave in flight.
+constexpr int VOCAB_ROWS_PER_WAVE = 4;
+__global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const float* __restrict__ x,
+                                                         const float* __restrict__ wte, float* __restrict__ logits) {
+  extern __shared__ float xs[];
+  for (int c = threadIdx.x; c < (d >> 2); c += WG) st4(xs + 4 * c, ld4(x + 4 * c));
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int v0 = (blockIdx.x * NWAVE + wave) * VOCAB_ROWS_PER_WAVE;
+  float acc[VOCAB_ROWS_PER_WAVE];
+#pragma unroll
+  for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) acc[r] = 0.f;
+  for (int c = lane; c < (d >> 2); c += 64) {
+    const float4 xv = ld4(xs + 4 * c);
+#pragma unroll
+    for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+      if (v0 + r < V) {
+        const float4 w = ld4(wte + (size_t)(v0 + r) * d + 4 * c);
+        acc[r] += (xv.x * w.x + xv.y * w.y) + (xv.z * w.z + xv.w * w.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+    const float s = wave_sum(acc[r]);
+    if (lane == 0 && v0 + r < V) logits[v0 + r] = s;
+  }
+}
+
+// AttentionBlock's formatQ + fusedWeights + softmax + attentionValues
+// (instructions.js:1129-1136, 1167-1176, 618-663, 1205-1212) for one (head, query
+// row) per workgroup, reading K and V rows 0..p of a [ctx, ldkv] cache. Masked
+// positions j > p get weight exactly 0 in the reference (exp(-1e9 - max) underflows),
+// so they are skipped rather than multiplied by zero.
+__global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk, float scale, const float* __restrict__ q,
+                                                        int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
+                                                        int ldkv, float* __restrict__ out, int ldo) {
+  extern __shared__ float scores[];
+  __shared__ float qs[256];
+  __shared__ float red[1024];
+  __shared__ float sh[NWAVE];
+  const int h = blockIdx.x, i = blockIdx.y;
+  const int nkeys = pos0 + i + 1;
+  const int tid = threadIdx.x;
+  if (tid < hs) qs[tid] = q[(size_t)i * ldq + h * hs + tid];
+  __syncthreads();
+  const int sub = tid & (lpk - 1), grp = tid / lpk, ngrp = WG / lpk;
+  const bool act = sub * 4 < hs;
+  const float4 qv = act ? ld4(qs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+  const float* kbase = Kc + h * hs + sub * 4;
+  const float* vbase = Vc + h * hs + sub * 4;
+  for (int j0 = 0; j0 < nkeys; j0 += ngrp) {
+    const int j = j0 + grp;
+    float part = 0.f;
+    if (act && j < nkeys) {
+      const float4 kv = ld4(kbase + (size_t)j * ldkv);
+      part = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
+    }
+    for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
+    if (sub == 0 && j < nkeys) scores[j] = part * scale;
+  }
+  __syncthreads();
+  float m = -3.402823e+38f;
+  for (int j = tid; j < nkeys; j += WG) m = fmaxf(m, scores[j]);
+  m = block_max(m, sh);
+  float s = 0.f;
+  for (int j = tid; j < nkeys; j += WG) {
+    const float e = expf(scores[j] - m);
+    scores[j] = e;
+    s += e;
+  }
+  s = block_sum(s, sh);
+  for (int j = tid; j < nkeys; j += WG) scores[j] = scores[j] / s;
+  __syncthreads();
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (act) {
+    for (int j = grp; j < nkeys; j += ngrp) fma4(acc, scores[j], ld4(vbase + (size_t)j * ldkv));
+    st4(red + grp * hs + sub * 4, acc);
+  }
+  __syncthreads();
+  if (tid < hs) {
+    float o = 0.f;
+    for (int g = 0; g < ngrp; ++g) o += red[g * hs + tid];
+    out[(size_t)i * ldo + h * hs + tid] = o;
+  }
+}
+
+__global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* __restrict__ src, int lds,
+                                                        float* __restrict__ dst, int ldd) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * WG + threadIdx.x;
+  if (c < cols4) st4(dst + (size_t)r * ldd + 4 * c, ld4(src + (size_t)r * lds + 4 * c));
+}
+
+// Greedy selection: selectTopK with top_k = 1 (globals.js:66-74) is a stable
+// descending sort, i.e. the largest logit with the lowest index on ties.
+__global__ __launch_bounds__(1024) void argmax_kernel(int V, const float* __restrict__ logits, int32_t* tok, int32_t* out,
+                                                       int slot) {
+  __shared__ float bv[1024];
+  __shared__ int bi[1024];
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int i = threadIdx.x; i < V; i += 1024) {
+    const float v = logits[i];
+    if (v > best || besti == 0x7fffffff) {
+      best = v;
+      besti = i;
+    }
+  }
+  bv[threadIdx.x] = best;
+  bi[threadIdx.x] = besti;
+  __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) {
+      const float ov = bv[threadIdx.x + s];
+      const int oi = bi[threadIdx.x + s];
+      const float cv = bv[threadIdx.x];
+      const int ci = bi[threadIdx.x];
+      if (oi != 0x7fffffff && (ci == 0x7fffffff || ov > cv || (ov == cv && oi < ci))) {
+        bv[threadIdx.x] = ov;
+        bi[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    tok[0] = bi[0];
+    if (out) out[slot] = bi[0];
+  }
+}
+
+inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+}  // namespace
+
+size_t gemv_workspace_floats(int M, int N, int K) {
+  return (size_t)cdiv(K, GEMV_KCHUNK) * (size_t)(M < 1 ? 1 : M) * (size_t)N;
+}
+
+hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
+                          float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  const int S = cdiv(K, GEMV_KCHUNK);
+  const dim3 grid(cdiv(N, 64), S);
+  switch (M) {
+    case 1: gemv_kn_partial<1><<<grid, WG, 0, s>>>(N, K, A, lda, W, ldw, workspace); break;
+    case 2: gemv_kn_partial<2><<<grid, WG, 0, s>>>(N, K, A, lda, W, ldw, workspace); break;
+    case 3: gemv_kn_partial<3><<<grid, WG, 0, s>>>(N, K, A, lda, W, ldw, workspace); break;
+    case 4: gemv_kn_partial<4><<<grid, WG, 0, s>>>(N, K, A, lda, W, ldw, workspace); break;
+    default: return hipErrorInvalidValue;
+  }
+  gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,
+                             const float* scale, const float* bias, float* C, int ldc, int epi, const float* resid,
+                             float* workspace, hipStream_t s) {
+  const int S = cdiv(K, GEMV_KCHUNK);
+  const dim3 grid(cdiv(N, 256), S);
+  switch (M) {
+    case 1: gemv_kn_i8_partial<1><<<grid, WG, 0, s>>>(N, K, A, lda, Wq, ldwq, scale, workspace); break;
+    case 2: gemv_kn_i8_partial<2><<<grid, WG, 0, s>>>(N, K, A, lda, Wq, ldwq, scale, workspace); break;
+    case 3: gemv_kn_i8_partial<3><<<grid, WG, 0, s>>>(N, K, A, lda, Wq, ldwq, scale, workspace); break;
+    case 4: gemv_kn_i8_partial<4><<<grid, WG, 0, s>>>(N, K, A, lda, Wq, ldwq, scale, workspace); break;
+    default: return hipErrorInvalidValue;
+  }
+  gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const float* scale, float* W, int ldw, hipStream_t s) {
+  dequant_i8_kernel<<<cdiv((size_t)K * (N >> 2), WG), WG, 0, s>>>(K, N, Wq, ldwq, scale, W, ldw);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
+                       float* C, int ldc, int epi, const float* resid, hipStream_t s) {
+  const dim3 grid(cdiv(N, 64), cdiv(M, 64));
+  gemm_tile64<<<grid, WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+  return hipGetLastError();
+}
+
+hipError_t launch_residual(size_t n4, const float* a, const float* b, float* out, hipStream_t s) {
+  residual_kernel<<<cdiv(n4, WG), WG, 0, s>>>(n4, a, b, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_gelu(size_t n4, const float* x, float* out, hipStream_t s) {
+  gelu_kernel<<<cdiv(n4, WG), WG, 0, s>>>(n4, x, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_layernorm(int M, int N, const float* x, int ldx, const float* gamma, const float* beta, float* out, int ldo,
+                            hipStream_t s) {
+  layernorm_kernel<<<M, WG, 0, s>>>(N, x, ldx, gamma, beta, out, ldo);
+  return hipGetLastError();
+}
+
+hipError_t launch_softmax(int M, int N, const float* x, float* out, hipStream_t s) {
+  softmax_kernel<<<M, WG, 0, s>>>(N, x, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_embed(const int32_t* idx, int T, int d, int pos0, const float* wte, const float* wpe, float* out, hipStream_t s) {
+  embed_kernel<<<T, WG, 0, s>>>(idx, d, pos0, wte, wpe, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, float* logits, hipStream_t s) {
+  const int rows_per_wg = NWAVE * VOCAB_ROWS_PER_WAVE;
+  vocab_gemv_kernel<<<cdiv(V, rows_per_wg), WG, sizeof(float) * d, s>>>(V, d, x, wte, logits);
+  return hipGetLastError();
+}
+
+hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
+                            const float* Vc, int ldkv, float* out, int ldo, hipStream_t s) {
+  int lpk = 1;
+  while (lpk * 4 < hs) lpk <<= 1;
+  if (lpk > 64 || hs > 256 || (hs & 3)) return hipErrorInvalidValue;
+  const size_t smem = sizeof(float) * (size_t)(pos0 + Tq);
+  if (smem > 48 * 1024) return hipErrorInvalidValue;
+  attention_kernel<<<dim3(H, Tq), WG, smem, s>>>(pos0, hs, lpk, scale, q, ldq, Kc, Vc, ldkv, out, ldo);
+  return hipGetLastError();
+}
+
+hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float* dst, int ldd, hipStream_t s) {
+  copy_rows_kernel<<<dim3(cdiv(cols >> 2, WG), rows), WG, 0, s>>>(cols >> 2, src, lds, dst, ldd);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax(int V, const float* logits, int32_t* tok, int32_t* out, int slot, hipStream_t s) {
+  argmax_kernel<<<1, 1024, 0, s>>>(V, logits, tok, out, slot);
+  return hipGetLastError();
+}
+
+}  // namespace wgpt

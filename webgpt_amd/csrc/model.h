@@ -1,0 +1,57 @@
+// Device-side state of one loaded model.
+#ifndef WGPT_MODEL_H
+#define WGPT_MODEL_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <vector>
+
+#include "../../include/webgpt_amd.h"
+
+namespace wgpt {
+
+// One linear layer's weight: fp32 [K,N], or int8 words [K,N/4] + per-column scale [N].
+struct LinW {
+  float* w = nullptr;
+  int32_t* q = nullptr;
+  float* s = nullptr;
+};
+
+struct LayerW {
+  float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
+  LinW attn, proj, fc, fc2;  // c_attn [d,3d], c_proj [d,d], c_fc [d,4d], mlp c_proj [4d,d]
+  float *attn_b = nullptr, *proj_b = nullptr, *fc_b = nullptr, *fc2_b = nullptr;
+};
+
+struct Model {
+  wgpt_params p{};
+  int L = 0, H = 0, d = 0, hs = 0, ctx = 0, V = 0, maxT = 0;
+  bool finalized = false;
+  int decode_mode = 0;
+  int pos = 0;     // positions held by the KV cache
+  int tap_T = 0;   // rows of the recorded taps (0 = none)
+
+  float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
+  std::vector<LayerW> layers;
+
+  float* kv = nullptr;  // [L][2][ctx][d]: keys then values of each layer
+  // activations for up to maxT rows
+  float *x = nullptr, *ln = nullptr, *qkv = nullptr, *att = nullptr, *tmp = nullptr, *h = nullptr;
+  float* logits = nullptr;       // [V]
+  float* part = nullptr;         // GEMV partial sums
+  float* dq = nullptr;           // fp32 scratch for a dequantised int8 matrix (prefill)
+  float* taps = nullptr;         // [(2+6L)][maxT][d]
+  int32_t* tok_dev = nullptr;    // [maxT] token ids of the current call
+  int32_t* out_tok_dev = nullptr;  // [ctx] ids chosen by the greedy loop
+
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  float last_ms = 0.f;
+  std::vector<void*> allocs;
+};
+
+void destroy_all_models();
+
+}  // namespace wgpt
+
+#endif

@@ -1,0 +1,450 @@
+// Whole-model entry points: GPT.loadModel (model.js:270-488) becomes
+// wgpt_model_create / set_tensor / finalize, GPT.run (model.js:104-268) becomes
+// wgpt_prefill (whole window) and wgpt_decode (window extended by one token, served
+// from a device-resident KV cache).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+#include "kernels.h"
+#include "model.h"
+
+namespace wgpt {
+
+static std::unordered_map<wgpt_model, Model*>& models() {
+  static std::unordered_map<wgpt_model, Model*> m;
+  return m;
+}
+static wgpt_model g_next_model = 1;
+
+static Model* find_model(wgpt_model h) {
+  auto it = models().find(h);
+  if (it == models().end()) {
+    fail(WGPT_ERR_ARG, "unknown model handle %llu", (unsigned long long)h);
+    return nullptr;
+  }
+  return it->second;
+}
+
+static int dev_alloc(Model* m, size_t bytes, void** out) {
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes + 16);
+  if (e != hipSuccess) return fail(WGPT_ERR_NOMEM, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  m->allocs.push_back(p);
+  *out = p;
+  return WGPT_OK;
+}
+
+// One named tensor of the weight directory: where it goes and how big it must be.
+struct Slot {
+  void** dst;
+  size_t bytes;
+};
+
+static bool parse_name(Model* m, const std::string& name, Slot* slot) {
+  const size_t d = m->d, L = m->L;
+  const size_t f = sizeof(float);
+  if (name == "transformer.wte.weight") { *slot = {(void**)&m->wte, (size_t)m->V * d * f}; return true; }
+  if (name == "transformer.wpe.weight") { *slot = {(void**)&m->wpe, (size_t)m->ctx * d * f}; return true; }
+  if (name == "transformer.ln_f.weight") { *slot = {(void**)&m->lnf_g, d * f}; return true; }
+  if (name == "transformer.ln_f.bias") { *slot = {(void**)&m->lnf_b, d * f}; return true; }
+  const char* prefix = "transformer.h.";
+  if (name.compare(0, strlen(prefix), prefix) != 0) return false;
+  size_t pos = strlen(prefix), end = name.find('.', pos);
+  if (end == std::string::npos || end == pos) return false;
+  size_t li = 0;
+  for (size_t i = pos; i < end; ++i) {
+    if (name[i] < '0' || name[i] > '9') return false;
+    li = li * 10 + (size_t)(name[i] - '0');
+    if (li >= L) return false;
+  }
+  LayerW& l = m->layers[li];
+  const std::string rest = name.substr(end + 1);
+  struct Lin { const char* stem; LinW* w; float** bias; size_t K, N; };
+  const Lin lins[4] = {{"attn.c_attn", &l.attn, &l.attn_b, d, 3 * d},
+                       {"attn.c_proj", &l.proj, &l.proj_b, d, d},
+                       {"mlp.c_fc", &l.fc, &l.fc_b, d, 4 * d},
+                       {"mlp.c_proj", &l.fc2, &l.fc2_b, 4 * d, d}};
+  if (rest == "ln_1.weight") { *slot = {(void**)&l.ln1_g, d * f}; return true; }
+  if (rest == "ln_1.bias") { *slot = {(void**)&l.ln1_b, d * f}; return true; }
+  if (rest == "ln_2.weight") { *slot = {(void**)&l.ln2_g, d * f}; return true; }
+  if (rest == "ln_2.bias") { *slot = {(void**)&l.ln2_b, d * f}; return true; }
+  for (const Lin& ln : lins) {
+    const std::string stem = ln.stem;
+    if (rest == stem + ".bias") { *slot = {(void**)ln.bias, ln.N * f}; return true; }
+    if (m->p.weight_dtype == 0) {
+      if (rest == stem + ".weight") { *slot = {(void**)&ln.w->w, ln.K * ln.N * f}; return true; }
+    } else {
+      if (rest == stem + ".weight.q") { *slot = {(void**)&ln.w->q, ln.K * (ln.N / 4) * sizeof(int32_t)}; return true; }
+      if (rest == stem + ".weight.scale") { *slot = {(void**)&ln.w->s, ln.N * f}; return true; }
+    }
+  }
+  return false;
+}
+
+// C[M,ldc] = epi(A . W + bias) with W fp32 or int8 weight-only.
+static int linear(Model* m, int M, int N, int K, const float* A, int lda, const LinW& w, const float* bias, float* C,
+                  int ldc, int epi, const float* resid) {
+  hipStream_t s = rt().stream;
+  hipError_t e;
+  if (w.q) {
+    if (M <= GEMV_MAX_ROWS) {
+      e = launch_gemv_kn_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
+    } else {
+      e = launch_dequant_i8(K, N, w.q, N / 4, w.s, m->dq, N, s);
+      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, s);
+    }
+  } else if (M <= GEMV_MAX_ROWS) {
+    e = launch_gemv_kn(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
+  } else {
+    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, s);
+  }
+  if (e != hipSuccess) return fail(WGPT_ERR_HIP, "linear layer launch: %s", hipGetErrorString(e));
+  return WGPT_OK;
+}
+
+#define LAUNCH(call)                                                                          \
+  do {                                                                                        \
+    hipError_t e_ = (call);                                                                   \
+    if (e_ != hipSuccess) return fail(WGPT_ERR_HIP, "%s: %s", #call, hipGetErrorString(e_));  \
+  } while (0)
+
+static int tap(Model* m, int T, size_t index, const float* src) {
+  if (!m->taps) return WGPT_OK;
+  WGPT_HIP(hipMemcpyAsync(m->taps + index * (size_t)T * m->d, src, sizeof(float) * (size_t)T * m->d,
+                          hipMemcpyDeviceToDevice, rt().stream));
+  return WGPT_OK;
+}
+
+// The forward of model.js:118-240 for T tokens at positions pos0..pos0+T-1, one
+// kernel (or two) per instruction block. Token ids are in m->tok_dev.
+static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
+  hipStream_t s = rt().stream;
+  const int d = m->d, H = m->H, hs = m->hs, hid = 4 * d;
+  const float scale = (float)(1.0 / std::sqrt((double)hs));  // model.js:321
+  const bool taps = want_taps && m->taps;
+  size_t ti = 0;
+  int rc;
+  LAUNCH(launch_embed(m->tok_dev, T, d, pos0, m->wte, m->wpe, m->x, s));
+  if (taps && (rc = tap(m, T, ti, m->x))) return rc;
+  ++ti;
+  for (int li = 0; li < m->L; ++li) {
+    const LayerW& l = m->layers[li];
+    float* Kc = m->kv + ((size_t)li * 2 + 0) * m->ctx * d;
+    float* Vc = m->kv + ((size_t)li * 2 + 1) * m->ctx * d;
+    LAUNCH(launch_layernorm(T, d, m->x, d, l.ln1_g, l.ln1_b, m->ln, d, s));
+    if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
+    ++ti;
+    if ((rc = linear(m, T, 3 * d, d, m->ln, d, l.attn, l.attn_b, m->qkv, 3 * d, EPI_NONE, nullptr))) return rc;
+    LAUNCH(launch_copy_rows(T, d, m->qkv + d, 3 * d, Kc + (size_t)pos0 * d, d, s));
+    LAUNCH(launch_copy_rows(T, d, m->qkv + 2 * d, 3 * d, Vc + (size_t)pos0 * d, d, s));
+    LAUNCH(launch_attention(T, pos0, H, hs, scale, m->qkv, 3 * d, Kc, Vc, d, m->att, d, s));
+    if (taps) {
+      if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->tmp, d, EPI_NONE, nullptr))) return rc;
+      if ((rc = tap(m, T, ti, m->tmp))) return rc;
+      LAUNCH(launch_residual((size_t)T * d / 4, m->tmp, m->x, m->x, s));
+    } else {
+      if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->x, d, EPI_RESIDUAL, m->x))) return rc;
+    }
+    ++ti;
+    if (taps && (rc = tap(m, T, ti, m->x))) return rc;
+    ++ti;
+    LAUNCH(launch_layernorm(T, d, m->x, d, l.ln2_g, l.ln2_b, m->ln, d, s));
+    if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
+    ++ti;
+    if ((rc = linear(m, T, hid, d, m->ln, d, l.fc, l.fc_b, m->h, hid, EPI_GELU, nullptr))) return rc;
+    if (taps) {
+      if ((rc = linear(m, T, d, hid, m->h, hid, l.fc2, l.fc2_b, m->tmp, d, EPI_NONE, nullptr))) return rc;
+      if ((rc = tap(m, T, ti, m->tmp))) return rc;
+      LAUNCH(launch_residual((size_t)T * d / 4, m->tmp, m->x, m->x, s));
+    } else {
+      if ((rc = linear(m, T, d, hid, m->h, hid, l.fc2, l.fc2_b, m->x, d, EPI_RESIDUAL, m->x))) return rc;
+    }
+    ++ti;
+    if (taps && (rc = tap(m, T, ti, m->x))) return rc;
+    ++ti;
+  }
+  if (taps) {
+    LAUNCH(launch_layernorm(T, d, m->x, d, m->lnf_g, m->lnf_b, m->ln, d, s));
+    if ((rc = tap(m, T, ti, m->ln))) return rc;
+    LAUNCH(launch_vocab_gemv(m->V, d, m->ln + (size_t)(T - 1) * d, m->wte, m->logits, s));
+  } else {
+    // Only the last row is de-embedded (instructions.js:849-856).
+    LAUNCH(launch_layernorm(1, d, m->x + (size_t)(T - 1) * d, d, m->lnf_g, m->lnf_b, m->ln, d, s));
+    LAUNCH(launch_vocab_gemv(m->V, d, m->ln, m->wte, m->logits, s));
+  }
+  return WGPT_OK;
+}
+
+static int finish_timed(Model* m, float* logits) {
+  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
+  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  return WGPT_OK;
+}
+
+static void destroy_model(Model* m) {
+  for (void* p : m->allocs) (void)hipFree(p);
+  if (m->ev0) (void)hipEventDestroy(m->ev0);
+  if (m->ev1) (void)hipEventDestroy(m->ev1);
+  delete m;
+}
+
+void destroy_all_models() {
+  for (auto& kv : models()) destroy_model(kv.second);
+  models().clear();
+}
+
+}  // namespace wgpt
+
+using namespace wgpt;
+
+extern "C" {
+
+int wgpt_model_create(const wgpt_params* p, wgpt_model* out) {
+  WGPT_REQUIRE_INIT();
+  if (!p || !out) return fail(WGPT_ERR_ARG, "wgpt_model_create: NULL argument");
+  if (p->n_layer < 1 || p->n_head < 1 || p->n_embd < 1 || p->n_ctx < 1 || p->vocab_size < 1)
+    return fail(WGPT_ERR_ARG, "wgpt_model_create: all of n_layer, n_head, n_embd, n_ctx, vocab_size must be positive");
+  // model.js:294-297
+  if (p->n_embd % 4 != 0) return fail(WGPT_ERR_ARG, "Model load failed: n_embd must be divisible by 4.");
+  if (p->n_embd % p->n_head != 0) return fail(WGPT_ERR_ARG, "Model load failed: n_embd must be divisible by n_head.");
+  if ((p->n_embd / p->n_head) % 4 != 0) return fail(WGPT_ERR_ARG, "Model load failed: n_embd / n_head must be divisible by 4.");
+  if (p->n_embd % 8 != 0) return fail(WGPT_ERR_ARG, "Cols must be divisible by 16.");  // FastMatMul on [*, n_embd]
+  if (p->n_embd / p->n_head > 256) return fail(WGPT_ERR_ARG, "wgpt_model_create: head size above 256 is not supported");
+  if (p->n_ctx > 12288) return fail(WGPT_ERR_ARG, "wgpt_model_create: n_ctx above 12288 is not supported");
+  if (p->weight_dtype != 0 && p->weight_dtype != 1) return fail(WGPT_ERR_ARG, "wgpt_model_create: weight_dtype must be 0 (fp32) or 1 (int8)");
+  if (p->max_prefill < 0 || p->max_prefill > p->n_ctx) return fail(WGPT_ERR_ARG, "wgpt_model_create: max_prefill must be in [0, n_ctx]");
+  Model* m = new Model();
+  m->p = *p;
+  m->L = p->n_layer; m->H = p->n_head; m->d = p->n_embd; m->ctx = p->n_ctx; m->V = p->vocab_size;
+  m->hs = m->d / m->H;
+  m->maxT = p->max_prefill ? p->max_prefill : p->n_ctx;
+  m->layers.resize(m->L);
+  *out = g_next_model++;
+  models()[*out] = m;
+  return WGPT_OK;
+}
+
+int wgpt_model_set_tensor(wgpt_model h, const char* name, const void* data, size_t bytes) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (m->finalized) return fail(WGPT_ERR_STATE, "wgpt_model_set_tensor: model already finalised");
+  if (!name || !data) return fail(WGPT_ERR_ARG, "wgpt_model_set_tensor: NULL argument");
+  Slot slot;
+  if (!parse_name(m, name, &slot)) return fail(WGPT_ERR_ARG, "wgpt_model_set_tensor: unknown tensor name '%s'", name);
+  if (bytes != slot.bytes) return fail(WGPT_ERR_ARG, "wgpt_model_set_tensor: '%s' needs %zu bytes, got %zu", name, slot.bytes, bytes);
+  if (!*slot.dst) {
+    int rc = dev_alloc(m, bytes, slot.dst);
+    if (rc) return rc;
+  }
+  WGPT_HIP(hipMemcpyAsync(*slot.dst, data, bytes, hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  return WGPT_OK;
+}
+
+int wgpt_model_finalize(wgpt_model h) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (m->finalized) return WGPT_OK;
+  const bool i8 = m->p.weight_dtype == 1;
+  if (!m->wte || !m->wpe || !m->lnf_g || !m->lnf_b) return fail(WGPT_ERR_STATE, "wgpt_model_finalize: embeddings or final layer norm missing");
+  for (int i = 0; i < m->L; ++i) {
+    const LayerW& l = m->layers[i];
+    const LinW* lw[4] = {&l.attn, &l.proj, &l.fc, &l.fc2};
+    bool ok = l.ln1_g && l.ln1_b && l.ln2_g && l.ln2_b && l.attn_b && l.proj_b && l.fc_b && l.fc2_b;
+    for (const LinW* w : lw) ok = ok && (i8 ? (w->q && w->s) : (w->w != nullptr));
+    if (!ok) return fail(WGPT_ERR_STATE, "wgpt_model_finalize: layer %d is missing tensors", i);
+  }
+  const size_t d = m->d, T = m->maxT, f = sizeof(float);
+  int rc;
+  if ((rc = dev_alloc(m, (size_t)m->L * 2 * m->ctx * d * f, (void**)&m->kv))) return rc;
+  if ((rc = dev_alloc(m, T * d * f, (void**)&m->x))) return rc;
+  if ((rc = dev_alloc(m, T * d * f, (void**)&m->ln))) return rc;
+  if ((rc = dev_alloc(m, T * 3 * d * f, (void**)&m->qkv))) return rc;
+  if ((rc = dev_alloc(m, T * d * f, (void**)&m->att))) return rc;
+  if ((rc = dev_alloc(m, T * d * f, (void**)&m->tmp))) return rc;
+  if ((rc = dev_alloc(m, T * 4 * d * f, (void**)&m->h))) return rc;
+  if ((rc = dev_alloc(m, (size_t)m->V * f, (void**)&m->logits))) return rc;
+  if ((rc = dev_alloc(m, T * sizeof(int32_t), (void**)&m->tok_dev))) return rc;
+  if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
+  size_t ws = gemv_workspace_floats(GEMV_MAX_ROWS, 4 * (int)d, (int)d);
+  const size_t ws2 = gemv_workspace_floats(GEMV_MAX_ROWS, (int)d, 4 * (int)d);
+  if (ws2 > ws) ws = ws2;
+  if ((rc = dev_alloc(m, ws * f, (void**)&m->part))) return rc;
+  if (i8 && (rc = dev_alloc(m, d * 4 * d * f, (void**)&m->dq))) return rc;
+  if ((m->p.flags & WGPT_FLAG_TAPS) && (rc = dev_alloc(m, (size_t)(2 + 6 * m->L) * T * d * f, (void**)&m->taps))) return rc;
+  WGPT_HIP(hipMemsetAsync(m->kv, 0, (size_t)m->L * 2 * m->ctx * d * f, rt().stream));
+  WGPT_HIP(hipEventCreate(&m->ev0));
+  WGPT_HIP(hipEventCreate(&m->ev1));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  m->pos = 0;
+  m->finalized = true;
+  return WGPT_OK;
+}
+
+int wgpt_prefill(wgpt_model h, const int32_t* tokens, int T, float* logits) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_prefill: model not finalised");
+  if (!tokens || T < 1) return fail(WGPT_ERR_ARG, "wgpt_prefill: tokens and T >= 1 required");
+  if (T > m->maxT) return fail(WGPT_ERR_ARG, "wgpt_prefill: T = %d exceeds max_prefill = %d", T, m->maxT);
+  for (int i = 0; i < T; ++i)
+    if (tokens[i] < 0 || tokens[i] >= m->V) return fail(WGPT_ERR_ARG, "wgpt_prefill: token id %d at %d outside [0, %d)", tokens[i], i, m->V);
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, tokens, sizeof(int32_t) * (size_t)T, hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
+  m->pos = 0;
+  m->tap_T = 0;
+  int rc = forward_blocks(m, T, 0, true);
+  if (rc) return rc;
+  rc = finish_timed(m, logits);
+  if (rc) return rc;
+  m->pos = T;
+  m->tap_T = m->taps ? T : 0;
+  return WGPT_OK;
+}
+
+int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode: model not finalised");
+  if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode: token id %d outside [0, %d)", token, m->V);
+  if (m->pos >= m->ctx) return fail(WGPT_ERR_STATE, "wgpt_decode: context of %d positions is full; prefill a slid window", m->ctx);
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
+  int rc = forward_blocks(m, 1, m->pos, false);
+  if (rc) return rc;
+  rc = finish_timed(m, logits);
+  if (rc) return rc;
+  m->pos += 1;
+  return WGPT_OK;
+}
+
+int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_tokens, float* logits) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: model not finalised");
+  if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: token id %d outside [0, %d)", token, m->V);
+  if (steps < 1 || !out_tokens) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: steps >= 1 and out_tokens required");
+  if (m->pos + steps > m->ctx)
+    return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
+  for (int i = 0; i < steps; ++i) {
+    int rc = forward_blocks(m, 1, m->pos + i, false);
+    if (rc) return rc;
+    LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
+  }
+  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
+  WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_tok_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
+  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  m->pos += steps;
+  return WGPT_OK;
+}
+
+int wgpt_model_reset_cache(wgpt_model h) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  m->pos = 0;
+  m->tap_T = 0;
+  return WGPT_OK;
+}
+
+int wgpt_model_position(wgpt_model h, int* pos) {
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (pos) *pos = m->pos;
+  return WGPT_OK;
+}
+
+int wgpt_model_tap(wgpt_model h, const char* name, float* out, size_t n_floats) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!name || !out) return fail(WGPT_ERR_ARG, "wgpt_model_tap: NULL argument");
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_model_tap: model not finalised");
+  const std::string n = name;
+  const size_t d = m->d;
+  const float* src = nullptr;
+  size_t count = 0;
+  int layer = -1;
+  char which[16] = "";
+  if (sscanf(name, "kv%d_%15s", &layer, which) == 2 && layer >= 0 && layer < m->L && (!strcmp(which, "k") || !strcmp(which, "v"))) {
+    src = m->kv + ((size_t)layer * 2 + (which[0] == 'v' ? 1 : 0)) * m->ctx * d;
+    count = (size_t)m->pos * d;
+  } else {
+    if (!m->taps || m->tap_T == 0) return fail(WGPT_ERR_STATE, "wgpt_model_tap: no taps recorded (WGPT_FLAG_TAPS and a prefill are needed)");
+    const size_t T = m->tap_T;
+    long index = -1;
+    if (n == "tok_pos_emb") index = 0;
+    else if (n == "ln_f") index = 1 + 6 * (long)m->L;
+    else if (sscanf(name, "block%d_%15s", &layer, which) == 2 && layer >= 0 && layer < m->L) {
+      const char* subs[6] = {"ln1", "attn", "r1", "ln2", "mlp", "r2"};
+      for (int k = 0; k < 6; ++k)
+        if (!strcmp(which, subs[k])) index = 1 + 6 * (long)layer + k;
+    }
+    if (index < 0) return fail(WGPT_ERR_ARG, "wgpt_model_tap: unknown tap '%s'", name);
+    src = m->taps + (size_t)index * T * d;
+    count = T * d;
+  }
+  if (n_floats != count) return fail(WGPT_ERR_ARG, "wgpt_model_tap: '%s' holds %zu floats, caller asked for %zu", name, count, n_floats);
+  if (count == 0) return WGPT_OK;
+  WGPT_HIP(hipMemcpyAsync(out, src, sizeof(float) * count, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  return WGPT_OK;
+}
+
+int wgpt_model_last_gpu_ms(wgpt_model h, float* ms) {
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (ms) *ms = m->last_ms;
+  return WGPT_OK;
+}
+
+int wgpt_model_decode_bytes(wgpt_model h, int t, uint64_t* bytes) {
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (t < 0 || t > m->ctx) return fail(WGPT_ERR_ARG, "wgpt_model_decode_bytes: t outside [0, n_ctx]");
+  const uint64_t d = m->d, L = m->L, V = m->V;
+  uint64_t w;
+  if (m->p.weight_dtype == 0) w = 4 * (L * (12 * d * d + 13 * d) + V * d + 2 * d);
+  else w = L * (12 * d * d) + 4 * (L * (13 * d + 9 * d) + V * d + 2 * d);
+  if (bytes) *bytes = w + 8 * L * d * (uint64_t)t;
+  return WGPT_OK;
+}
+
+int wgpt_model_set_decode_mode(wgpt_model h, int mode) {
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (mode != 0) return fail(WGPT_ERR_ARG, "wgpt_model_set_decode_mode: mode %d is not available", mode);
+  m->decode_mode = mode;
+  return WGPT_OK;
+}
+
+int wgpt_model_destroy(wgpt_model h) {
+  WGPT_REQUIRE_INIT();
+  auto it = models().find(h);
+  if (it == models().end()) return fail(WGPT_ERR_ARG, "wgpt_model_destroy: unknown model handle %llu", (unsigned long long)h);
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  destroy_model(it->second);
+  models().erase(it);
+  return WGPT_OK;
+}
+
+}  // extern "C"

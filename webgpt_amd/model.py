@@ -1,0 +1,229 @@
+"""GPT: the driver class of the reference's model.js over the HIP library.
+
+`initialize()` loads a weight directory (params_gpt.json + one little-endian f32
+`<tensor>_gpt.bin` per tensor, model.js:270-488) or takes tensors from memory;
+`run(idx)` returns the logits of the last token of the window `idx`
+(model.js:104-268); `generate()` is the sampling loop of model.js:53-102.
+
+Two execution routes exist for `run`:
+  - the whole-model entry points of the library (wgpt_prefill / wgpt_decode), which
+    keep a KV cache on the device and are used whenever `idx` is the previous
+    window plus one token;
+  - `run_blocks(idx)`, which builds the reference's pass list block by block
+    (model.js:118-240) and replays it, recomputing the whole window.
+"""
+import ctypes as C
+import json
+import math
+import os
+import time
+
+import numpy as np
+
+from . import _lib, blocks, sampling
+from .blocks import (AttentionBlock, DeEmbedBlock, EmbedBlock, FastMatMulBlock, GeluBlock, LayerNormBlock,
+                     ResidualBlock, SoftmaxBlock)
+
+_FP = C.POINTER(C.c_float)
+_IP = C.POINTER(C.c_int32)
+
+
+class GPT:
+    def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0):
+        self.folder = folder
+        self.tokenizerType = type
+        self.initialized = False
+        self.device = None
+        self.model = None
+        self.tokenizer = tokenizer
+        self.params = None
+        self.externalBuffer = None
+        self.unloadDeletionStack = []
+        self.defaultPrompt = None
+        self.defaultTopK = None
+        self.defaultTemperature = None
+        self.defaultTokens = None
+        self._tensors = tensors
+        self._params_in = params
+        self._flags = flags
+        self._device_index = device_index
+        self._handle = None
+        self._history = []
+        self.lastGpuMs = 0.0
+
+    # ---------------- lifecycle ----------------
+
+    def initialize(self):
+        if self.initialized:
+            print("Model already initialized")
+            return
+        self.device = blocks.Device(self._device_index)  # raises if no gfx950 device: "WebGPU is not supported"
+        blocks.initializeOperations(self.device)
+        self.model, self.params = self.loadModel(self.folder)
+        if self.tokenizerType == "bpe":
+            self.defaultPrompt = "What is the answer to life, the universe, and everything?\n"
+            self.defaultTopK, self.defaultTemperature, self.defaultTokens = 3, 1, 30
+        else:
+            self.defaultPrompt = "WILL:\nAh, how dare you challenge me?\nHave you forgotten I built WebGPT?\n"
+            self.defaultTopK, self.defaultTemperature, self.defaultTokens = 2, 1, 80
+        self.initialized = True
+
+    def loadParameters(self, weightsFolder):
+        """model.js:289-337."""
+        if self._params_in is not None:
+            params = dict(self._params_in)
+        else:
+            with open(os.path.join(weightsFolder, "params_gpt.json")) as f:
+                params = json.load(f)
+        if params["n_embd"] % 4 != 0:
+            raise ValueError("Model load failed: n_embd must be divisible by 4.")
+        if params["n_embd"] % params["n_head"] != 0:
+            raise ValueError("Model load failed: n_embd must be divisible by n_head.")
+        if (params["n_embd"] // params["n_head"]) % 4 != 0:
+            raise ValueError("Model load failed: n_embd / n_head must be divisible by 4.")
+        # The vocabulary is never split here: one buffer, one launch.
+        params["vocab_chunk_size"] = params["vocab_size"]
+        params["vocab_chunk_instances"] = 1
+        params["head_size"] = params["n_embd"] // params["n_head"]
+        params["hidden_size"] = params["n_embd"] * 4
+        params["attention_scale"] = 1 / math.sqrt(params["n_embd"] / params["n_head"])
+        params["bias"] = params.get("bias", True)
+        return params
+
+    def _fetch(self, weightsFolder, name):
+        if self._tensors is not None:
+            return self._tensors[name]
+        return np.fromfile(os.path.join(weightsFolder, name + "_gpt.bin"), dtype="<f4")
+
+    def loadModel(self, folder):
+        if self.initialized:
+            print("Model already loaded")
+            return None
+        weightsFolder = folder
+        params = self.loadParameters(weightsFolder)
+        names = sorted(self._tensors) if self._tensors is not None else None
+        int8 = names is not None and any(n.endswith(".weight.q") for n in names)
+        p = _lib.Params(params["n_layer"], params["n_head"], params["n_embd"], params["n_ctx"], params["vocab_size"],
+                        1 if int8 else 0, params.get("max_prefill", 0), self._flags)
+        h = C.c_uint64(0)
+        _lib.call("wgpt_model_create", C.byref(p), C.byref(h))
+        self._handle = h.value
+        if names is None:
+            names = [n for n in self._directory_names(params)]
+        for n in names:
+            a = np.ascontiguousarray(self._fetch(weightsFolder, n))
+            _lib.call("wgpt_model_set_tensor", self._handle, n.encode(), a.ctypes.data_as(C.c_void_p), a.nbytes)
+        _lib.call("wgpt_model_finalize", self._handle)
+        return {"handle": self._handle}, params
+
+    @staticmethod
+    def _directory_names(params):
+        yield "transformer.wte.weight"
+        yield "transformer.wpe.weight"
+        for i in range(params["n_layer"]):
+            for s in ("ln_1.weight", "ln_1.bias", "attn.c_attn.weight", "attn.c_attn.bias", "attn.c_proj.weight",
+                      "attn.c_proj.bias", "ln_2.weight", "ln_2.bias", "mlp.c_fc.weight", "mlp.c_fc.bias",
+                      "mlp.c_proj.weight", "mlp.c_proj.bias"):
+                yield f"transformer.h.{i}.{s}"
+        yield "transformer.ln_f.weight"
+        yield "transformer.ln_f.bias"
+
+    def unloadBuffers(self):
+        for b in self.unloadDeletionStack:
+            b.destroy()
+        self.unloadDeletionStack = []
+        if self._handle is not None:
+            _lib.call("wgpt_model_destroy", self._handle)
+            self._handle = None
+        self.initialized = False
+
+    def initTensor(self, data, dims, ops=("storage",)):
+        buf = blocks.init_tensor(data, dims, ops)
+        self.unloadDeletionStack.append(buf)
+        return buf
+
+    def bufferSize(self, dimX, dimY=1, dimZ=1):
+        return dimX * dimY * dimZ * 4
+
+    # ---------------- forward ----------------
+
+    def prefill(self, idx):
+        ids = np.ascontiguousarray(idx, dtype=np.int32)
+        logits = np.empty(self.params["vocab_size"], np.float32)
+        _lib.call("wgpt_prefill", self._handle, ids.ctypes.data_as(_IP), len(ids), logits.ctypes.data_as(_FP))
+        self._history = [int(t) for t in ids]
+        self._update_ms()
+        return logits
+
+    def decode(self, token):
+        logits = np.empty(self.params["vocab_size"], np.float32)
+        _lib.call("wgpt_decode", self._handle, int(token), logits.ctypes.data_as(_FP))
+        self._history.append(int(token))
+        self._update_ms()
+        return logits
+
+    def decode_greedy(self, token, steps, want_logits=False):
+        out = np.empty(steps, np.int32)
+        logits = np.empty(self.params["vocab_size"], np.float32) if want_logits else None
+        _lib.call("wgpt_decode_greedy", self._handle, int(token), steps, out.ctypes.data_as(_IP),
+                  logits.ctypes.data_as(_FP) if want_logits else None)
+        self._history += [int(token)] + [int(t) for t in out[:-1]]
+        self._update_ms()
+        return (out, logits) if want_logits else out
+
+    def _update_ms(self):
+        ms = C.c_float(0)
+        _lib.call("wgpt_model_last_gpu_ms", self._handle, C.byref(ms))
+        self.lastGpuMs = ms.value
+
+    def run(self, idx):
+        """Logits of the last token of window `idx` (model.js:104). Served from the KV
+        cache when `idx` extends the previous window by one token, else recomputed."""
+        idx = [int(t) for t in idx]
+        if len(idx) == len(self._history) + 1 and len(idx) <= self.params["n_ctx"] and idx[:-1] == self._history \
+                and len(self._history) > 0:
+            return self.decode(idx[-1])
+        return self.prefill(idx)
+
+    def tap(self, name, rows=None):
+        d = self.params["n_embd"]
+        if rows is None:
+            pos = C.c_int(0)
+            _lib.call("wgpt_model_position", self._handle, C.byref(pos))
+            rows = pos.value
+        out = np.empty((rows, d), np.float32)
+        _lib.call("wgpt_model_tap", self._handle, name.encode(), out.ctypes.data_as(_FP), out.size)
+        return out
+
+    def decode_bytes(self, t):
+        b = C.c_uint64(0)
+        _lib.call("wgpt_model_decode_bytes", self._handle, int(t), C.byref(b))
+        return b.value
+
+    def set_decode_mode(self, mode):
+        _lib.call("wgpt_model_set_decode_mode", self._handle, int(mode))
+
+    def generate(self, prompt, max_new_tokens, top_k, temperature):
+        """The loop of model.js:53-102. `prompt` is a string when a tokenizer was
+        given, else a list of token ids; yields decoded text or ids accordingly."""
+        if not self.initialized:
+            print("Model not loaded yet")
+            return
+        history = list(self.tokenizer.encode(prompt)) if self.tokenizer else [int(t) for t in prompt]
+        warmupRuns = 3
+        totalTime = 0.0
+        n_ctx = self.params["n_ctx"]
+        for i in range(max_new_tokens):
+            idx_cond = history[-n_ctx:]
+            startTime = time.perf_counter()
+            logits = self.run(idx_cond)
+            lapsed = (time.perf_counter() - startTime) * 1000.0
+            if i >= warmupRuns:
+                totalTime += lapsed
+            sel = sampling.selectTopK(logits, top_k) if top_k != 1 else \
+                {"topKIndices": [int(np.argmax(logits))], "topKProbs": [float(np.max(logits))]}
+            probs = sampling.cpuSoftmax(sel["topKProbs"], temperature)
+            idx_next = sel["topKIndices"][sampling.sampleFromDistribution(probs)]
+            history = history + [idx_next]
+            yield self.tokenizer.decode([idx_next]) if self.tokenizer else idx_next
+        self.averageMs = totalTime / max(1, max_new_tokens - warmupRuns)
