@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-token forward path: GPT-2 117M fp32 batch-1 greedy decode.
+
+One "step" is one decode token: the whole forward of one new token against the
+device-resident KV cache, followed by the on-device arg-max that feeds the next
+step. Weights, KV cache and the first token are resident in HBM when the timed
+region starts; nothing crosses PCIe inside it. Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config gpt2-117m]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+
+
+def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
+    """The CPU restatement of the reference's kernels (oracle/), run the way the
+    reference runs: every token recomputes the whole window (model.js:69,104)."""
+    from oracle import ref
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_weights
+    from webgpt_amd import synth
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    hist = [int(t) for t in prompt]
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 8 and (time.perf_counter() - t_all) < budget_s:
+        t0 = time.perf_counter()
+        logits = ref.forward(p, w, np.array(hist, np.int32))
+        times.append(time.perf_counter() - t0)
+        hist.append(int(np.argmax(logits)))
+    ms = 1000.0 * float(np.mean(times))
+    return {"value": round(ms, 3), "unit": "ms/token", "cores": ref.get_threads(), "kind": "port",
+            "sample": f"{len(times)} greedy tokens after a {len(prompt)}-token prompt, whole window recomputed per "
+                      f"token as GPT.run does, C restatement of the WGSL kernels with OpenMP"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=253)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="gpt2-117m")
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--mode", type=int, default=None, help="decode implementation (default: library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (batch-1 decode does not shard usefully); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from webgpt_amd import synth
+    from webgpt_amd.model import GPT
+
+    cfg = dict(synth.CONFIGS[args.config])
+    if cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
+        print(f"bench.py: prompt {cfg['prompt']} + warmup + steps exceeds n_ctx {cfg['n_ctx']}", file=sys.stderr)
+        sys.exit(2)
+    tensors = dict(synth.make_tensors(cfg, args.seed))
+    prompt = synth.make_prompt(cfg, args.seed)
+    gpt = GPT(None, "bpe", tensors=tensors, params=synth.model_params(cfg))
+    gpt.initialize()
+    if args.mode is not None:
+        gpt.set_decode_mode(args.mode)
+
+    # prefill (untimed for the headline; reported separately)
+    gpt.prefill(prompt)  # first call also loads the code objects
+    t0 = time.perf_counter()
+    logits = gpt.prefill(prompt)
+    prefill_wall_ms = (time.perf_counter() - t0) * 1000.0
+    prefill_gpu_ms = gpt.lastGpuMs
+    tok = int(np.argmax(logits))
+
+    # warmup steps, then exactly K timed steps, all on the device
+    pos = len(prompt)
+    if args.warmup > 0:
+        ids = gpt.decode_greedy(tok, args.warmup)
+        tok = int(ids[-1])
+        pos += args.warmup
+    gpt.device.sync()
+    t0 = time.perf_counter()
+    ids = gpt.decode_greedy(tok, args.steps)
+    gpt.device.sync()
+    wall_ms = (time.perf_counter() - t0) * 1000.0
+    gpu_ms = gpt.lastGpuMs
+    ms_per_step = wall_ms / args.steps
+    bytes_total = sum(gpt.decode_bytes(pos + i) for i in range(args.steps))
+    achieved = bytes_total / (gpu_ms * 1e-3) / 1e9
+
+    # per-token host loop with logits read-back (what GPT.run returns), PCIe inclusive
+    per_tok = []
+    nxt = int(ids[-1])
+    for _ in range(min(32, cfg["n_ctx"] - pos - args.steps)):
+        t0 = time.perf_counter()
+        lg = gpt.decode(nxt)
+        per_tok.append((time.perf_counter() - t0) * 1000.0)
+        nxt = int(np.argmax(lg))
+
+    out = {
+        "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
+                  else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
+        "value": round(ms_per_step, 5),
+        "unit": "ms/token",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if cfg["dtype"] == "f32" else "f32 activations, int8 weights",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: L{cfg['n_layer']} H{cfg['n_head']} d{cfg['n_embd']} V{cfg['vocab_size']}, "
+                               f"prompt {cfg['prompt']}, greedy decode, context {pos}..{pos + args.steps - 1}",
+                   "seed": args.seed},
+        "tokens_per_s": round(1000.0 / ms_per_step, 1),
+        "gpu_ms_per_token": round(gpu_ms / args.steps, 5),
+        "prefill_tokens_per_s": round(len(prompt) / (prefill_gpu_ms * 1e-3), 1),
+        "prefill_ms": round(prefill_gpu_ms, 3),
+        "prefill_wall_ms": round(prefill_wall_ms, 3),
+        "host_loop_ms_per_token": {"mean": round(float(np.mean(per_tok)), 4), "p50": round(float(np.median(per_tok)), 4),
+                                   "note": "wgpt_decode per token incl. logits read-back over PCIe"} if per_tok else None,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "one decode token (all launches of the token)",
+                     "bytes_per_step": int(bytes_total / args.steps)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt)
+    gpt.unloadBuffers()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -110,7 +110,7 @@ def test_deembed_ragged_vocab(device):
     assert close(got, want), worst(got, want)
 
 
-@pytest.mark.parametrize("T,H,hs", [(1, 2, 8), (15, 4, 32), (64, 6, 64), (130, 12, 64), (5, 1, 4), (33, 25, 64)])
+@pytest.mark.parametrize("T,H,hs", [(1, 2, 8), (15, 4, 32), (64, 6, 64), (130, 12, 64), (5, 2, 4), (33, 25, 64)])
 def test_attention(device, T, H, hs):
     d = H * hs
     x = rnd(T, d)
