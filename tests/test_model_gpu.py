@@ -140,3 +140,38 @@ def test_gpt2_117m_shape_prefill_and_decode(device):
     assert greedy_ok(got, want)
     assert gpt.decode_bytes(0) == 4 * (12 * (12 * 768 * 768 + 13 * 768) + 50257 * 768 + 2 * 768)
     gpt.unloadBuffers()
+
+
+@pytest.mark.parametrize("name,steps", [("toy", 40), ("gpt2-117m", 6)])
+def test_persistent_decode_matches_per_block_decode_and_oracle(device, name, steps):
+    # decode mode 1 (one persistent kernel per token) against mode 0 (one kernel per block) and the oracle
+    cfg = dict(synth.CONFIGS[name])
+    gpt, tensors = load(cfg, seed=5, random_ln=(name == "toy"))
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(8, "prompt", 10 + steps, cfg["vocab_size"])
+    out = {}
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        gpt.prefill(tokens[:10])
+        out[mode] = [gpt.decode(int(tokens[10 + i])) for i in range(steps)]
+    for i in range(steps):
+        assert close(out[1][i], out[0][i]), (i, worst(out[1][i], out[0][i]))
+    for i in (0, steps - 1):
+        want = ref.forward(p, w, tokens[: 11 + i])
+        assert close(out[1][i], want), (i, worst(out[1][i], want))
+        assert greedy_ok(out[1][i], want)
+    # the cache written by the persistent kernel serves the per-block path and vice versa
+    gpt.set_decode_mode(1)
+    gpt.prefill(tokens[:10])
+    a = gpt.decode(int(tokens[10]))
+    gpt.set_decode_mode(0)
+    b = gpt.decode(int(tokens[11]))
+    assert close(a, out[0][0]) and close(b, out[0][1])
+    # multi-step greedy launch: ids equal the per-block greedy loop
+    ids = {}
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        lg = gpt.prefill(tokens[:10])
+        ids[mode] = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), min(steps, 24))]
+    assert ids[0] == ids[1]
+    gpt.unloadBuffers()

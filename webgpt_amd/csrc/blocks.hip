@@ -260,7 +260,7 @@ int wgpt_attention(int T, int d, float scale, int H, int hs, wgpt_buf x, wgpt_bu
   if ((rc = matmul_dev(T, d, d, px, wq, pbq, Q))) return rc;
   if ((rc = matmul_dev(T, d, d, px, wk, pbk, Km))) return rc;
   if ((rc = matmul_dev(T, d, d, px, wv, pbv, Vm))) return rc;
-  hipError_t e = launch_attention(T, 0, H, hs, scale, Q, d, Km, Vm, d, O, d, rt().stream);
+  hipError_t e = launch_attention(T, 0, H, hs, scale, Q, d, Km, Vm, (size_t)hs, d, O, d, rt().stream);
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "attention launch: %s", hipGetErrorString(e));
   return matmul_dev(T, d, d, O, wo, pbo, po);
 }

@@ -1,0 +1,71 @@
+// Host interface of the whole-token persistent decode kernel.
+#ifndef WGPT_DECODE_PERSISTENT_H
+#define WGPT_DECODE_PERSISTENT_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace wgpt {
+
+constexpr int PD_THREADS = 512;
+
+// How one linear layer is split over the workgroups: workgroup w finishes columns
+// [w*cpw, (w+1)*cpw) of N; a column is S segments of 256 contraction elements; the
+// cpw*S items of a workgroup are dealt to its waves in runs of ipw.
+struct PhaseGeom {
+  int N, cpw, S, ipw;
+};
+
+// Offsets (in floats) inside one layer's block of small parameters:
+// [c_attn bias 3d | attn c_proj bias d | c_fc bias 4d | mlp c_proj bias d | ln1 g,b | ln2 g,b].
+struct LayerParamOffsets {
+  int bA, bC, bD, bE, ln1g, ln1b, ln2g, ln2b, stride;
+};
+__host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
+  LayerParamOffsets o;
+  o.bA = 0; o.bC = 3 * d; o.bD = 4 * d; o.bE = 8 * d;
+  o.ln1g = 9 * d; o.ln1b = 10 * d; o.ln2g = 11 * d; o.ln2b = 12 * d;
+  o.stride = 13 * d;
+  return o;
+}
+
+struct PersistentArgs {
+  int L, H, d, hs, ctx, V;
+  int G;      // workgroups in the grid (one per compute unit)
+  int split;  // position slices per head in the attention phase
+  float scale;
+  PhaseGeom gA, gC, gD, gE;
+  int rows_per_wg;  // vocabulary rows per workgroup
+  int xs_floats, attp_floats, part_floats;  // LDS carve-up
+  // slab-layout weights of all layers in one allocation: layer l starts at
+  // slabs + l*slab_stride; c_attn at 0, then attn c_proj, c_fc, mlp c_proj (float4 units)
+  const float4* slabs;
+  size_t slab_stride, slab_offC, slab_offD, slab_offE;
+  const float* lparams;  // [L][13d] small per-layer parameters (LayerParamOffsets)
+  const float *wte, *wpe, *lnf_g, *lnf_b;
+  float* kv;  // [L][2][H][ctx][hs]
+  // {value, epoch} exchange buffers
+  unsigned long long *bufQKV, *bufATT, *bufR1, *bufH, *bufR2, *bufAM;
+  float* logits;
+  const int32_t* tok;  // tok[0]: token of the first step
+  int32_t* out_tok;    // [nsteps] arg-max of each step
+  int* err;            // set non-zero when a bounded wait expired
+  unsigned ebase;      // epoch of the last word published by earlier launches
+  int pos0, nsteps;
+};
+
+PhaseGeom make_geom(int N, int K, int G);
+size_t slab_float4s(const PhaseGeom& g, int G);
+// Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g.
+hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, int G, float4* slab, hipStream_t s);
+int persistent_max_items(const PersistentArgs& a);
+size_t persistent_lds_bytes(const PersistentArgs& a);
+// Epochs consumed by one decode step.
+inline unsigned persistent_epochs_per_step(int L) { return 5u * (unsigned)L + 1u; }
+hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s);
+
+}  // namespace wgpt
+
+#endif

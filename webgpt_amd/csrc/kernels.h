@@ -42,9 +42,12 @@ hipError_t launch_embed(const int32_t* idx, int T, int d, int pos0, const float*
 // logits[v] = x . wte[v,:]
 hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, float* logits, hipStream_t s);
 // Causal attention of Tq query rows (absolute positions pos0..pos0+Tq-1) against
-// keys/values 0..pos of a [ctx, d]-shaped cache. q row i is at q + i*ldq + h*hs.
+// keys/values 0..pos. q row i is at q + i*ldq + h*hs; key row j of head h is at
+// Kc + h*hstride + j*ldkv (likewise values).
 hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
-                            const float* Vc, int ldkv, float* out, int ldo, hipStream_t s);
+                            const float* Vc, size_t hstride, int ldkv, float* out, int ldo, hipStream_t s);
+// Appends the K and V columns of qkv[T,3d] at positions pos0.. of a head-major cache [H][ctx][hs].
+hipError_t launch_kv_append(int T, int d, int hs, int ctx, int pos0, const float* qkv, float* Kc, float* Vc, hipStream_t s);
 // Copies rows of src (row stride lds, `cols` floats wide) to dst (row stride ldd).
 hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float* dst, int ldd, hipStream_t s);
 // tok[0] = argmax(logits[0..V)) with the lowest index on ties; also stored to out[slot].

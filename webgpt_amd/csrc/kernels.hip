@@ -370,12 +370,12 @@ __global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const floa
 
 // AttentionBlock's formatQ + fusedWeights + softmax + attentionValues
 // (instructions.js:1129-1136, 1167-1176, 618-663, 1205-1212) for one (head, query
-// row) per workgroup, reading K and V rows 0..p of a [ctx, ldkv] cache. Masked
+// row) per workgroup, reading K and V rows 0..p of head h at Kc + h*hstride + j*ldkv. Masked
 // positions j > p get weight exactly 0 in the reference (exp(-1e9 - max) underflows),
 // so they are skipped rather than multiplied by zero.
 __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk, float scale, const float* __restrict__ q,
                                                         int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
-                                                        int ldkv, float* __restrict__ out, int ldo) {
+                                                        size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
   extern __shared__ float scores[];
   __shared__ float qs[256];
   __shared__ float red[1024];
@@ -388,8 +388,8 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   const int sub = tid & (lpk - 1), grp = tid / lpk, ngrp = WG / lpk;
   const bool act = sub * 4 < hs;
   const float4 qv = act ? ld4(qs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-  const float* kbase = Kc + h * hs + sub * 4;
-  const float* vbase = Vc + h * hs + sub * 4;
+  const float* kbase = Kc + h * hstride + sub * 4;
+  const float* vbase = Vc + h * hstride + sub * 4;
   for (int j0 = 0; j0 < nkeys; j0 += ngrp) {
     const int j = j0 + grp;
     float part = 0.f;
@@ -431,6 +431,19 @@ __global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* _
   const int r = blockIdx.y;
   const int c = blockIdx.x * WG + threadIdx.x;
   if (c < cols4) st4(dst + (size_t)r * ldd + 4 * c, ld4(src + (size_t)r * lds + 4 * c));
+}
+
+// Appends T rows of keys and values (columns d..2d and 2d..3d of qkv[T,3d]) to the
+// head-major cache: row (h, pos0+i) of K at Kc + (h*ctx + pos0+i)*hs.
+__global__ __launch_bounds__(WG) void kv_append_kernel(int d, int hs, int ctx, int pos0, const float* __restrict__ qkv,
+                                                        float* __restrict__ Kc, float* __restrict__ Vc) {
+  const int i = blockIdx.x;
+  for (int c4 = threadIdx.x; c4 < (d >> 2); c4 += WG) {
+    const int c = c4 * 4, h = c / hs, e = c - h * hs;
+    const size_t dst = ((size_t)h * ctx + pos0 + i) * hs + e;
+    st4(Kc + dst, ld4(qkv + (size_t)i * 3 * d + d + c));
+    st4(Vc + dst, ld4(qkv + (size_t)i * 3 * d + 2 * d + c));
+  }
 }
 
 // Greedy selection: selectTopK with top_k = 1 (globals.js:66-74) is a stable
@@ -554,18 +567,23 @@ hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, flo
 }
 
 hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
-                            const float* Vc, int ldkv, float* out, int ldo, hipStream_t s) {
+                            const float* Vc, size_t hstride, int ldkv, float* out, int ldo, hipStream_t s) {
   int lpk = 1;
   while (lpk * 4 < hs) lpk <<= 1;
   if (lpk > 64 || hs > 256 || (hs & 3)) return hipErrorInvalidValue;
   const size_t smem = sizeof(float) * (size_t)(pos0 + Tq);
   if (smem > 48 * 1024) return hipErrorInvalidValue;
-  attention_kernel<<<dim3(H, Tq), WG, smem, s>>>(pos0, hs, lpk, scale, q, ldq, Kc, Vc, ldkv, out, ldo);
+  attention_kernel<<<dim3(H, Tq), WG, smem, s>>>(pos0, hs, lpk, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
   return hipGetLastError();
 }
 
 hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float* dst, int ldd, hipStream_t s) {
   copy_rows_kernel<<<dim3(cdiv(cols >> 2, WG), rows), WG, 0, s>>>(cols >> 2, src, lds, dst, ldd);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_append(int T, int d, int hs, int ctx, int pos0, const float* qkv, float* Kc, float* Vc, hipStream_t s) {
+  kv_append_kernel<<<T, WG, 0, s>>>(d, hs, ctx, pos0, qkv, Kc, Vc);
   return hipGetLastError();
 }
 

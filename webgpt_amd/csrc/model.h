@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/webgpt_amd.h"
+#include "decode_persistent.h"
 
 namespace wgpt {
 
@@ -35,7 +36,7 @@ struct Model {
   float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
   std::vector<LayerW> layers;
 
-  float* kv = nullptr;  // [L][2][ctx][d]: keys then values of each layer
+  float* kv = nullptr;  // [L][2][H][ctx][hs]: keys then values of each layer, head-major
   // activations for up to maxT rows
   float *x = nullptr, *ln = nullptr, *qkv = nullptr, *att = nullptr, *tmp = nullptr, *h = nullptr;
   float* logits = nullptr;       // [V]
@@ -44,6 +45,12 @@ struct Model {
   float* taps = nullptr;         // [(2+6L)][maxT][d]
   int32_t* tok_dev = nullptr;    // [maxT] token ids of the current call
   int32_t* out_tok_dev = nullptr;  // [ctx] ids chosen by the greedy loop
+
+  // persistent whole-token decode (decode_mode 1): slab-layout weights, exchange buffers
+  bool persist_ok = false;
+  PersistentArgs pa{};
+  int* perr = nullptr;       // device error word of the persistent kernel
+  unsigned epoch = 0;        // last epoch published by earlier launches
 
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   float last_ms = 0.f;

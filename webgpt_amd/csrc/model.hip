@@ -140,9 +140,8 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
     if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
     ++ti;
     if ((rc = linear(m, T, 3 * d, d, m->ln, d, l.attn, l.attn_b, m->qkv, 3 * d, EPI_NONE, nullptr))) return rc;
-    LAUNCH(launch_copy_rows(T, d, m->qkv + d, 3 * d, Kc + (size_t)pos0 * d, d, s));
-    LAUNCH(launch_copy_rows(T, d, m->qkv + 2 * d, 3 * d, Vc + (size_t)pos0 * d, d, s));
-    LAUNCH(launch_attention(T, pos0, H, hs, scale, m->qkv, 3 * d, Kc, Vc, d, m->att, d, s));
+    LAUNCH(launch_kv_append(T, d, hs, m->ctx, pos0, m->qkv, Kc, Vc, s));
+    LAUNCH(launch_attention(T, pos0, H, hs, scale, m->qkv, 3 * d, Kc, Vc, (size_t)m->ctx * hs, hs, m->att, d, s));
     if (taps) {
       if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->tmp, d, EPI_NONE, nullptr))) return rc;
       if ((rc = tap(m, T, ti, m->tmp))) return rc;
@@ -176,6 +175,118 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
     // Only the last row is de-embedded (instructions.js:849-856).
     LAUNCH(launch_layernorm(1, d, m->x + (size_t)(T - 1) * d, d, m->lnf_g, m->lnf_b, m->ln, d, s));
     LAUNCH(launch_vocab_gemv(m->V, d, m->ln, m->wte, m->logits, s));
+  }
+  return WGPT_OK;
+}
+
+// Prepares the persistent whole-token decode path: slab-layout copies of the linear
+// weights, the per-layer pointer table and the exchange buffers. Leaves
+// m->persist_ok false (and the per-block path in charge) for shapes it does not cover.
+static int setup_persistent(Model* m) {
+  m->persist_ok = false;
+  const int d = m->d, hid = 4 * d, G = 256, split = 4;
+  if (m->p.weight_dtype != 0 || m->hs != 64) return WGPT_OK;
+  if (rt().compute_units < G) return WGPT_OK;
+  PersistentArgs& a = m->pa;
+  a = PersistentArgs{};
+  a.L = m->L; a.H = m->H; a.d = d; a.hs = m->hs; a.ctx = m->ctx; a.V = m->V;
+  a.G = G; a.split = split;
+  a.scale = (float)(1.0 / std::sqrt((double)m->hs));
+  a.gA = make_geom(3 * d, d, G);
+  a.gC = make_geom(d, d, G);
+  a.gD = make_geom(hid, d, G);
+  a.gE = make_geom(d, hid, G);
+  a.rows_per_wg = (m->V + G - 1) / G;
+  const int attw = m->H * split * (m->hs + 2);
+  if (persistent_max_items(a) > 16 || hid > 8192 || attw > 8192 || m->H * split > G) return WGPT_OK;
+  if (((m->ctx + split - 1) / split + 31) / 32 > 8) return WGPT_OK;
+  a.xs_floats = a.gE.S * 256;
+  a.attp_floats = attw > 2 * G ? attw : 2 * G;
+  int pf = 8 * (m->hs + 4);
+  const int cpw_max = a.gD.cpw > a.gA.cpw ? a.gD.cpw : a.gA.cpw;
+  if (cpw_max * 8 > pf) pf = cpw_max * 8;
+  a.part_floats = pf;
+  if (persistent_lds_bytes(a) > 150 * 1024) return WGPT_OK;
+
+  int rc;
+  // all slabs in one allocation, all small per-layer parameters in another
+  a.slab_offC = slab_float4s(a.gA, G);
+  a.slab_offD = a.slab_offC + slab_float4s(a.gC, G);
+  a.slab_offE = a.slab_offD + slab_float4s(a.gD, G);
+  a.slab_stride = a.slab_offE + slab_float4s(a.gE, G);
+  float4* slabs;
+  if ((rc = dev_alloc(m, a.slab_stride * (size_t)m->L * sizeof(float4), (void**)&slabs))) return rc;
+  const LayerParamOffsets po = layer_param_offsets(d);
+  float* lparams;
+  if ((rc = dev_alloc(m, sizeof(float) * (size_t)po.stride * m->L, (void**)&lparams))) return rc;
+  for (int i = 0; i < m->L; ++i) {
+    const LayerW& l = m->layers[i];
+    float4* sl = slabs + (size_t)i * a.slab_stride;
+    LAUNCH(build_slab(l.attn.w, 3 * d, d, a.gA, G, sl, rt().stream));
+    LAUNCH(build_slab(l.proj.w, d, d, a.gC, G, sl + a.slab_offC, rt().stream));
+    LAUNCH(build_slab(l.fc.w, hid, d, a.gD, G, sl + a.slab_offD, rt().stream));
+    LAUNCH(build_slab(l.fc2.w, d, hid, a.gE, G, sl + a.slab_offE, rt().stream));
+    float* lp = lparams + (size_t)i * po.stride;
+    const struct { int off; const float* src; int n; } parts[8] = {
+        {po.bA, l.attn_b, 3 * d}, {po.bC, l.proj_b, d}, {po.bD, l.fc_b, hid}, {po.bE, l.fc2_b, d},
+        {po.ln1g, l.ln1_g, d},    {po.ln1b, l.ln1_b, d}, {po.ln2g, l.ln2_g, d}, {po.ln2b, l.ln2_b, d}};
+    for (const auto& pt : parts)
+      WGPT_HIP(hipMemcpyAsync(lp + pt.off, pt.src, sizeof(float) * pt.n, hipMemcpyDeviceToDevice, rt().stream));
+  }
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  a.slabs = slabs;
+  a.lparams = lparams;
+  a.wte = m->wte; a.wpe = m->wpe; a.lnf_g = m->lnf_g; a.lnf_b = m->lnf_b;
+  a.kv = m->kv;
+  const size_t words = (size_t)3 * d + attw + d + hid + d + 2 * G;
+  unsigned long long* buf;
+  if ((rc = dev_alloc(m, words * sizeof(unsigned long long), (void**)&buf))) return rc;
+  WGPT_HIP(hipMemsetAsync(buf, 0, words * sizeof(unsigned long long), rt().stream));
+  a.bufQKV = buf;
+  a.bufATT = a.bufQKV + 3 * d;
+  a.bufR1 = a.bufATT + attw;
+  a.bufH = a.bufR1 + d;
+  a.bufR2 = a.bufH + hid;
+  a.bufAM = a.bufR2 + d;
+  if ((rc = dev_alloc(m, sizeof(int), (void**)&m->perr))) return rc;
+  WGPT_HIP(hipMemsetAsync(m->perr, 0, sizeof(int), rt().stream));
+  a.logits = m->logits;
+  a.tok = m->tok_dev;
+  a.out_tok = m->out_tok_dev;
+  a.err = m->perr;
+  m->epoch = 0;
+  m->persist_ok = true;
+  return WGPT_OK;
+}
+
+// Runs `steps` greedy decode steps from position m->pos with the persistent kernel.
+// The first token is in m->tok_dev[0]; chosen ids land in m->out_tok_dev.
+static int decode_persistent(Model* m, int steps) {
+  PersistentArgs a = m->pa;
+  const unsigned per_step = persistent_epochs_per_step(m->L);
+  if (m->epoch > 0xffffffffu - per_step * (unsigned)steps - 8u) {
+    // epoch counter about to wrap: start over from clean exchange buffers
+    const size_t words = (size_t)(a.bufAM + 2 * a.G - a.bufQKV);
+    WGPT_HIP(hipMemsetAsync(a.bufQKV, 0, words * sizeof(unsigned long long), rt().stream));
+    m->epoch = 0;
+  }
+  a.ebase = m->epoch;
+  a.pos0 = m->pos;
+  a.nsteps = steps;
+  LAUNCH(launch_decode_persistent(a, rt().stream));
+  m->epoch += per_step * (unsigned)steps;
+  return WGPT_OK;
+}
+
+// After the stream has drained: did a bounded wait of the persistent kernel expire?
+static int check_persistent(Model* m) {
+  int herr = 0;
+  WGPT_HIP(hipMemcpy(&herr, m->perr, sizeof(int), hipMemcpyDeviceToHost));
+  if (herr != 0) {
+    (void)hipMemset(m->perr, 0, sizeof(int));
+    m->persist_ok = false;  // do not trust the exchange buffers again
+    m->decode_mode = 0;
+    return fail(WGPT_ERR_DEVICE, "persistent decode kernel: a bounded wait expired at epoch %d; the persistent path is now disabled", herr);
   }
   return WGPT_OK;
 }
@@ -285,6 +396,8 @@ int wgpt_model_finalize(wgpt_model h) {
   WGPT_HIP(hipEventCreate(&m->ev0));
   WGPT_HIP(hipEventCreate(&m->ev1));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
+  if ((rc = setup_persistent(m))) return rc;
+  m->decode_mode = m->persist_ok ? 1 : 0;
   m->pos = 0;
   m->finalized = true;
   return WGPT_OK;
@@ -323,10 +436,11 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  int rc = forward_blocks(m, 1, m->pos, false);
+  int rc = m->decode_mode == 1 ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
+  if (m->decode_mode == 1 && (rc = check_persistent(m))) return rc;
   m->pos += 1;
   return WGPT_OK;
 }
@@ -343,16 +457,26 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  for (int i = 0; i < steps; ++i) {
-    int rc = forward_blocks(m, 1, m->pos + i, false);
+  const bool persistent = m->decode_mode == 1;
+  if (persistent) {
+    int rc = decode_persistent(m, steps);
     if (rc) return rc;
-    LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
+  } else {
+    for (int i = 0; i < steps; ++i) {
+      int rc = forward_blocks(m, 1, m->pos + i, false);
+      if (rc) return rc;
+      LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
+    }
   }
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_tok_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
   if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  if (persistent) {
+    int rc = check_persistent(m);
+    if (rc) return rc;
+  }
   m->pos += steps;
   return WGPT_OK;
 }
@@ -386,8 +510,16 @@ int wgpt_model_tap(wgpt_model h, const char* name, float* out, size_t n_floats) 
   int layer = -1;
   char which[16] = "";
   if (sscanf(name, "kv%d_%15s", &layer, which) == 2 && layer >= 0 && layer < m->L && (!strcmp(which, "k") || !strcmp(which, "v"))) {
-    src = m->kv + ((size_t)layer * 2 + (which[0] == 'v' ? 1 : 0)) * m->ctx * d;
+    // the cache is head-major [H][ctx][hs]: gather rows 0..pos-1 into [pos, d]
     count = (size_t)m->pos * d;
+    if (n_floats != count) return fail(WGPT_ERR_ARG, "wgpt_model_tap: '%s' holds %zu floats, caller asked for %zu", name, count, n_floats);
+    if (count == 0) return WGPT_OK;
+    const float* base = m->kv + ((size_t)layer * 2 + (which[0] == 'v' ? 1 : 0)) * m->ctx * d;
+    for (int h2 = 0; h2 < m->H; ++h2)
+      WGPT_HIP(hipMemcpy2DAsync(out + (size_t)h2 * m->hs, sizeof(float) * d, base + (size_t)h2 * m->ctx * m->hs,
+                                sizeof(float) * m->hs, sizeof(float) * m->hs, (size_t)m->pos, hipMemcpyDeviceToHost, rt().stream));
+    WGPT_HIP(hipStreamSynchronize(rt().stream));
+    return WGPT_OK;
   } else {
     if (!m->taps || m->tap_T == 0) return fail(WGPT_ERR_STATE, "wgpt_model_tap: no taps recorded (WGPT_FLAG_TAPS and a prefill are needed)");
     const size_t T = m->tap_T;
@@ -432,7 +564,10 @@ int wgpt_model_decode_bytes(wgpt_model h, int t, uint64_t* bytes) {
 int wgpt_model_set_decode_mode(wgpt_model h, int mode) {
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
-  if (mode != 0) return fail(WGPT_ERR_ARG, "wgpt_model_set_decode_mode: mode %d is not available", mode);
+  if (mode != 0 && mode != 1) return fail(WGPT_ERR_ARG, "wgpt_model_set_decode_mode: unknown mode %d", mode);
+  if (mode == 1 && !m->persist_ok)
+    return fail(WGPT_ERR_STATE, "wgpt_model_set_decode_mode: the persistent decode path is not available for this model "
+                                "(needs fp32 weights, head size 64, 256 compute units)");
   m->decode_mode = mode;
   return WGPT_OK;
 }
