@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libwebgpt_amd.so")
+# WEBGPT_AMD_LIB selects another build of the same library (e.g. a profiling build).
+LIB_PATH = os.environ.get("WEBGPT_AMD_LIB") or os.path.join(_HERE, "libwebgpt_amd.so")
 
 
 class WgptError(RuntimeError):

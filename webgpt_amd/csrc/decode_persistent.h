@@ -9,7 +9,10 @@
 
 namespace wgpt {
 
-constexpr int PD_THREADS = 512;
+constexpr int PD_THREADS = 512;  // threads per workgroup
+constexpr int PD_GRID = 256;     // workgroups: one per compute unit of an MI355X
+constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase
+constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
 // [w*cpw, (w+1)*cpw) of N; a column is S segments of 256 contraction elements; the
@@ -32,13 +35,9 @@ __host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
 }
 
 struct PersistentArgs {
-  int L, H, d, hs, ctx, V;
-  int G;      // workgroups in the grid (one per compute unit)
-  int split;  // position slices per head in the attention phase
+  int L, H, d, ctx, V;
   float scale;
-  PhaseGeom gA, gC, gD, gE;
   int rows_per_wg;  // vocabulary rows per workgroup
-  int xs_floats, attp_floats, part_floats;  // LDS carve-up
   // slab-layout weights of all layers in one allocation: layer l starts at
   // slabs + l*slab_stride; c_attn at 0, then attn c_proj, c_fc, mlp c_proj (float4 units)
   const float4* slabs;
@@ -52,16 +51,17 @@ struct PersistentArgs {
   const int32_t* tok;  // tok[0]: token of the first step
   int32_t* out_tok;    // [nsteps] arg-max of each step
   int* err;            // set non-zero when a bounded wait expired
+  unsigned long long* trace;  // optional [G][512] clock samples of the last step (WGPT_TRACE builds), or null
   unsigned ebase;      // epoch of the last word published by earlier launches
   int pos0, nsteps;
 };
 
-PhaseGeom make_geom(int N, int K, int G);
-size_t slab_float4s(const PhaseGeom& g, int G);
+PhaseGeom make_geom(int N, int K);
+size_t slab_float4s(const PhaseGeom& g);
 // Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g.
-hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, int G, float4* slab, hipStream_t s);
-int persistent_max_items(const PersistentArgs& a);
-size_t persistent_lds_bytes(const PersistentArgs& a);
+hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4* slab, hipStream_t s);
+// Model shapes the persistent kernel is instantiated for.
+bool persistent_supports(int d, int n_head, int n_ctx);
 // Epochs consumed by one decode step.
 inline unsigned persistent_epochs_per_step(int L) { return 5u * (unsigned)L + 1u; }
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s);

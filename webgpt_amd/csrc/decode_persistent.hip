@@ -37,15 +37,21 @@ typedef unsigned long long u64;
 constexpr int NT = PD_THREADS;       // threads per workgroup
 constexpr int NW = NT / 64;          // waves per workgroup
 constexpr int SEG = 256;             // contraction elements per item (64 lanes x float4)
-#ifndef WGPT_NPMAX
-#define WGPT_NPMAX 8
-#endif
-constexpr int NPMAX = WGPT_NPMAX;   // a poll covers up to NPMAX*NT words
+constexpr int NPMAX = 8;             // a poll round covers up to NPMAX*NT words
+constexpr int LNMAX = 4;             // LayerNorm parameters held per thread: d <= LNMAX*NT
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 
 __device__ __forceinline__ u64 ld_word(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_word(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void publish(u64* p, float v, unsigned epoch) { st_word(p, ((u64)epoch << 32) | __float_as_uint(v)); }
+
+// Streaming (non-temporal) 128-bit load: weights are read once per token and must
+// not displace the small hot data (parameters, instructions) from the caches.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld_stream(const float4* p) {
+  const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+  return make_float4(t.x, t.y, t.z, t.w);
+}
 
 // Returns v unchanged but opaque to the optimiser: address arithmetic built on the
 // result cannot be hoisted out of the enclosing loops and kept in registers for the
@@ -54,16 +60,51 @@ __device__ __forceinline__ int opaque(int v) {
   asm volatile("" : "+v"(v));
   return v;
 }
-
 // Same for a wave-uniform value held in a scalar register.
 __device__ __forceinline__ int opaque_s(int v) {
   asm volatile("" : "+s"(v));
   return v;
 }
 
+// One data-parallel-primitive step: v (+|max) the value of another lane selected by
+// CTRL, only in the rows of ROWS; lanes without a source contribute the identity.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROWS, 0xf, true));
+}
+template <int CTRL, int ROWS>
+__device__ __forceinline__ float dpp_max(float v) {
+  const int ninf = __float_as_int(-INFINITY);
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(ninf, __float_as_int(v), CTRL, ROWS, 0xf, false)));
+}
+
+// Sum over the 64 lanes, returned as a wave-uniform value. Row-wise inclusive scan
+// (row_shr 1,2,4,8), then lane 15 of each row into the next row (row_bcast15) and
+// lane 31 into the upper half (row_bcast31): lane 63 holds the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  v = dpp_add<0x111, 0xf>(v);
+  v = dpp_add<0x112, 0xf>(v);
+  v = dpp_add<0x114, 0xf>(v);
+  v = dpp_add<0x118, 0xf>(v);
+  v = dpp_add<0x142, 0xa>(v);
+  v = dpp_add<0x143, 0xc>(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = dpp_max<0x111, 0xf>(v);
+  v = dpp_max<0x112, 0xf>(v);
+  v = dpp_max<0x114, 0xf>(v);
+  v = dpp_max<0x118, 0xf>(v);
+  v = dpp_max<0x142, 0xa>(v);
+  v = dpp_max<0x143, 0xc>(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+// Sum over each row of 16 lanes, every lane of the row gets it (row rotations).
+__device__ __forceinline__ float row16_sum(float v) {
+  v = dpp_add<0x128, 0xf>(v);
+  v = dpp_add<0x124, 0xf>(v);
+  v = dpp_add<0x122, 0xf>(v);
+  v = dpp_add<0x121, 0xf>(v);
   return v;
 }
 
@@ -78,7 +119,7 @@ __device__ __forceinline__ float gelu_ref(float x) {  // instructions.js:718-727
 
 struct Shared {
   int bail;
-  float red[2 * NW];
+  float red[32];
   float red_idx[NW];
 };
 __shared__ Shared sh;
@@ -86,106 +127,132 @@ __shared__ Shared sh;
 // Has any thread of this workgroup given up on a bounded wait?
 __device__ __forceinline__ int bail_flag() { return __hip_atomic_load(&sh.bail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
-// Polls n {value, epoch} words until all carry `epoch`, storing the values to dst
-// (LDS). Works in chunks of NPMAX*NT words; all loads of a round are issued before
-// any is tested. Returns false after SPIN_LIMIT rounds or when another thread or
-// workgroup has already given up.
-__device__ __forceinline__ bool poll_words(const u64* __restrict__ buf, int n, unsigned epoch, float* dst, int* err) {
+// All vector-memory loads issued so far have completed (vmcnt = 0); the other
+// counters are left alone. Placed after each poll so that registers requested
+// before the poll are known to have landed on every control path.
+__device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// Compile-time geometry of one model shape: everything the phases index with is a
+// constant, so the per-phase code is loads, FMAs and a few scalar compares. (A wave
+// retires only one instruction every few cycles; index arithmetic on the critical
+// path of a phase costs as much as the hop between phases.)
+template <int D_, int H_>
+struct Shape {
+  static constexpr int D = D_, H = H_, HS = D_ / H_, HID = 4 * D_;
+  static constexpr int G = PD_GRID, SPLIT = PD_SPLIT;
+  static constexpr int SD = (D + SEG - 1) / SEG;      // segments of a D-long contraction
+  static constexpr int SH = (HID + SEG - 1) / SEG;    // segments of a HID-long contraction
+  static constexpr int ATTW = H * SPLIT * (HS + 2);   // words of the attention exchange buffer
+  static_assert(HS == 64, "the attention phase is laid out for head size 64");
+  static_assert(D <= LNMAX * NT, "LayerNorm parameter registers cover d <= 2048");
+};
+
+// One linear phase: N outputs from a K-long input.
+template <int N_, int K_>
+struct Phase {
+  static constexpr int N = N_, K = K_;
+  static constexpr int CPW = (N + PD_GRID - 1) / PD_GRID;  // columns per workgroup
+  static constexpr int S = (K + SEG - 1) / SEG;            // segments per column
+  static constexpr int ITEMS = CPW * S;                    // items per workgroup
+  static constexpr int IPW = (ITEMS + NW - 1) / NW;        // items per wave
+};
+
+// Polls N {value, epoch} words until all carry `epoch`, storing the values to dst
+// (LDS). All loads of a round are issued before any is tested. On SPIN_LIMIT rounds,
+// or when another thread or workgroup has already given up, raises sh.bail.
+template <int N>
+__device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err) {
+  constexpr int NP = (N + NT - 1) / NT;
   const int t = opaque(threadIdx.x);
-  bool ok = true;
-  for (int c0 = 0; c0 < n && ok; c0 += NPMAX * NT) {
-    const u64* src = buf + c0;
-    float* out = dst + c0;
-    const int m = n - c0;
-    unsigned pending = 0;
+  unsigned pending = 0;
 #pragma unroll
-    for (int i = 0; i < NPMAX; ++i)
-      if (t + i * NT < m) pending |= 1u << i;
-    unsigned spins = 0;
-    while (pending) {
-      u64 pk[NPMAX];
+  for (int i = 0; i < NP; ++i)
+    if (i * NT + NT <= N || t + i * NT < N) pending |= 1u << i;
+  unsigned spins = 0;
+  while (pending) {
+    u64 pk[NP];
 #pragma unroll
-      for (int i = 0; i < NPMAX; ++i)
-        if (pending & (1u << i)) pk[i] = ld_word((src + i * NT) + t);
+    for (int i = 0; i < NP; ++i)
+      if (pending & (1u << i)) pk[i] = ld_word(buf + i * NT + t);
 #pragma unroll
-      for (int i = 0; i < NPMAX; ++i)
-        if ((pending & (1u << i)) && (unsigned)(pk[i] >> 32) == epoch) {
-          out[t + i * NT] = __uint_as_float((unsigned)pk[i]);
-          pending &= ~(1u << i);
-        }
-      if (pending) {
-        ++spins;
-        if (spins > SPIN_LIMIT || bail_flag() ||
-            ((spins & 255u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
-          sh.bail = 1;
-          atomicCAS(err, 0, (int)epoch);
-          ok = false;
-          break;
-        }
+    for (int i = 0; i < NP; ++i)
+      if ((pending & (1u << i)) && (unsigned)(pk[i] >> 32) == epoch) {
+        dst[t + i * NT] = __uint_as_float((unsigned)pk[i]);
+        pending &= ~(1u << i);
+      }
+    if (pending) {
+      ++spins;
+      if (spins > SPIN_LIMIT || bail_flag() ||
+          ((spins & 255u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+        sh.bail = 1;
+        atomicCAS(err, 0, (int)epoch);
+        break;
       }
     }
   }
-  return ok;
 }
 
-// Registers of one phase's weight slab share: MAXI float4 per lane plus the bias of
-// the column this thread will finish.
+// Registers of one linear phase: this wave's share of the weight slab (MAXI float4
+// per lane), the bias of the column this thread finishes, and the LayerNorm
+// parameters of the elements this thread normalises (phases with a LayerNorm).
 template <int MAXI>
 struct WSet {
   float4 w[MAXI];
   float bias;
+  float g[LNMAX], b[LNMAX];
 };
 
-// Requests the slab share of this wave. Item j (column j / S, segment j % S of this
-// workgroup's columns) is 64 consecutive float4; wave v owns items [v*ipw, (v+1)*ipw).
-template <int MAXI>
-__device__ __forceinline__ void load_items(WSet<MAXI>& ws, const float4* __restrict__ slab, const PhaseGeom& g, int K,
-                                           const float* __restrict__ bias, int wg, int wave, int lane) {
-  const int col0 = wg * g.cpw;
-  int ncols = g.N - col0;
-  ncols = ncols > g.cpw ? g.cpw : ncols;
-  const int nitems = ncols > 0 ? ncols * g.S : 0;
-  const int ln = opaque(lane);
-  const float4* base = slab + (size_t)wg * g.cpw * g.S * 64;
-  int j = opaque_s(wave) * g.ipw;
-  int seg = j % g.S;
+// Requests the slab share of this wave: items [wave*IPW, wave*IPW + IPW) of the
+// workgroup's `nitems`; item j is 64 consecutive float4 (column j / S, segment j % S).
+template <class P, int MAXI>
+__device__ __forceinline__ void load_items(WSet<MAXI>& ws, const float4* __restrict__ slab, const float* __restrict__ bias,
+                                           int nitems, int wg, int wave, int lane) {
+  static_assert(P::IPW <= MAXI, "register set too small");
+  const float4* base = slab + ((size_t)wg * P::ITEMS + (size_t)wave * P::IPW) * 64 + opaque(lane);
+  const int j0 = opaque_s(wave) * P::IPW;
 #pragma unroll
-  for (int i = 0; i < MAXI; ++i) {
+  for (int i = 0; i < P::IPW; ++i) {
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (i < g.ipw && j < nitems && seg * SEG + ln * 4 < K) v = (base + (size_t)j * 64)[ln];
+    if (j0 + i < nitems) v = ld_stream(base + i * 64);
     ws.w[i] = v;
-    ++j;
-    if (++seg == g.S) seg = 0;
   }
-  ws.bias = ((int)threadIdx.x < ncols) ? bias[col0 + threadIdx.x] : 0.f;
+  const int t = opaque(threadIdx.x);
+  ws.bias = (t < P::CPW && wg * P::CPW + t < P::N) ? bias[wg * P::CPW + t] : 0.f;
+}
+
+// Requests the LayerNorm parameters of elements tid, tid+NT, ... of a D-wide row.
+template <int D, int MAXI>
+__device__ __forceinline__ void load_ln(WSet<MAXI>& ws, const float* __restrict__ gamma, const float* __restrict__ beta) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int k = 0; k < (D + NT - 1) / NT; ++k) {
+    const int e = t + k * NT;
+    ws.g[k] = e < D ? gamma[e] : 0.f;
+    ws.b[k] = e < D ? beta[e] : 0.f;
+  }
 }
 
 // Dot products of this wave's items with the input vector xs (LDS, zero padded up
 // to S*SEG). Per (column, wave) partial sums go to part[col*NW + wave].
-template <int MAXI>
-__device__ __forceinline__ void gemv_items(const WSet<MAXI>& ws, const float* xs, float* part, const PhaseGeom& g, int wg,
-                                           int wave, int lane) {
-  const int col0 = wg * g.cpw;
-  int ncols = g.N - col0;
-  ncols = ncols > g.cpw ? g.cpw : ncols;
-  const int nitems = ncols > 0 ? ncols * g.S : 0;
-  int j = opaque_s(wave) * g.ipw;
-  int col = j / g.S;
-  int seg = j - col * g.S;
+template <class P, int MAXI>
+__device__ __forceinline__ void gemv_items(const WSet<MAXI>& ws, const float* xs, float* part, int nitems, int wave, int lane) {
+  lane = opaque(lane);
+  const int j0 = opaque_s(wave) * P::IPW;
+  int col = j0 / P::S;
+  int seg = j0 - col * P::S;
   float acc = 0.f;
 #pragma unroll
-  for (int i = 0; i < MAXI; ++i) {
-    if (i < g.ipw && j < nitems) {
+  for (int i = 0; i < P::IPW; ++i) {
+    if (j0 + i < nitems) {
       const float4 x = *reinterpret_cast<const float4*>(xs + seg * SEG + lane * 4);
       const float4 w = ws.w[i];
       acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
-      if (seg == g.S - 1 || i == g.ipw - 1 || j == nitems - 1) {
+      if (seg == P::S - 1 || i == P::IPW - 1 || j0 + i == nitems - 1) {
         const float r = wave_sum(acc);
         if (lane == 0) part[col * NW + wave] = r;
         acc = 0.f;
       }
-      ++j;
-      if (++seg == g.S) {
+      if (++seg == P::S) {
         seg = 0;
         ++col;
       }
@@ -194,149 +261,204 @@ __device__ __forceinline__ void gemv_items(const WSet<MAXI>& ws, const float* xs
 }
 
 // Sum of the per-wave partials of local column c, in ascending wave order.
-__device__ __forceinline__ float column_sum(const float* part, const PhaseGeom& g, int c) {
-  c = opaque(c);
-  const int v0 = (c * g.S) / g.ipw;
-  int v1 = ((c + 1) * g.S - 1) / g.ipw;
+template <class P>
+__device__ __forceinline__ float column_sum(const float* part, int c) {
+  const int v0 = (c * P::S) / P::IPW;
+  int v1 = ((c + 1) * P::S - 1) / P::IPW;
   v1 = v1 > NW - 1 ? NW - 1 : v1;
   float s = 0.f;
   for (int v = v0; v <= v1; ++v) s += part[c * NW + v];
   return s;
 }
 
-// LayerNorm of xs[0..d) in place (instructions.js:451-550 semantics: biased
-// variance about the mean, eps inside the sqrt, true division).
-__device__ __forceinline__ void layernorm_lds(float* xs, int d, const float* __restrict__ gamma,
-                                              const float* __restrict__ beta) {
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+// LayerNorm of xs[0..D) in place (instructions.js:451-550 semantics: biased variance
+// about the mean, eps inside the sqrt, true division). Every wave derives the two
+// statistics itself from LDS, so only the write-back needs barriers. xs is zero
+// beyond D up to S*SEG.
+template <int D, int MAXI>
+__device__ __forceinline__ void layernorm_lds(float* xs, const WSet<MAXI>& ws, int lane) {
+  constexpr int S = (D + SEG - 1) / SEG;
+  float4 v[S];
   float s = 0.f;
-  for (int e = threadIdx.x; e < d; e += NT) s += xs[e];
-  s = wave_sum(s);
-  if (lane == 0) sh.red[wave] = s;
-  __syncthreads();
-  float tot = 0.f;
 #pragma unroll
-  for (int v = 0; v < NW; ++v) tot += sh.red[v];
-  const float mean = tot / (float)d;
-  float q = 0.f;
-  for (int e = threadIdx.x; e < d; e += NT) {
-    const float a = xs[e] - mean;
-    q += a * a;
+  for (int s2 = 0; s2 < S; ++s2) {
+    v[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
+    s += (v[s2].x + v[s2].y) + (v[s2].z + v[s2].w);
   }
-  q = wave_sum(q);
-  if (lane == 0) sh.red[NW + wave] = q;
-  __syncthreads();
-  float var = 0.f;
+  const float mean = wave_sum(s) / (float)D;
+  float q = 0.f;
 #pragma unroll
-  for (int v = 0; v < NW; ++v) var += sh.red[NW + v];
-  const float stdev = sqrtf(var / (float)d + 1e-5f);
-  for (int e = threadIdx.x; e < d; e += NT) xs[e] = gamma[e] * ((xs[e] - mean) / stdev) + beta[e];
+  for (int s2 = 0; s2 < S; ++s2) {
+    if (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D) {
+      const float a0 = v[s2].x - mean, a1 = v[s2].y - mean, a2 = v[s2].z - mean, a3 = v[s2].w - mean;
+      q += (a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3);
+    }
+  }
+  const float stdev = sqrtf(wave_sum(q) / (float)D + 1e-5f);
+  __syncthreads();  // every wave has read xs
+  const int t = opaque(threadIdx.x);
+#pragma unroll
+  for (int k = 0; k < (D + NT - 1) / NT; ++k) {
+    const int e = t + k * NT;
+    if (k * NT + NT <= D || e < D) xs[e] = ws.g[k] * ((xs[e] - mean) / stdev) + ws.b[k];
+  }
   __syncthreads();
 }
 
-template <int MAXI, int MAXKV>
+#ifdef WGPT_TRACE
+#define TRACE(slot)                                                                              \
+  do {                                                                                           \
+    if (a.trace && tid == 0 && step == a.nsteps - 1) a.trace[(size_t)wg * 512 + (slot)] = wall_clock64(); \
+  } while (0)
+#define TRACE5(k)                                                                                 \
+  do {                                                                                            \
+    if (a.trace && tid == 0 && step == a.nsteps - 1 && li == 5) a.trace[(size_t)wg * 512 + 400 + PH * 16 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define TRACE(slot) do {} while (0)
+#define TRACE5(k) do {} while (0)
+#endif
+
+// Linear phases of a layer, in execution order.
+enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
+
+template <class C>
+struct Phases {
+  typedef Phase<3 * C::D, C::D> A;   // c_attn
+  typedef Phase<C::D, C::D> Cc;      // attention c_proj
+  typedef Phase<C::HID, C::D> Dd;    // c_fc
+  typedef Phase<C::D, C::HID> E;     // mlp c_proj
+  static constexpr int MAXI = (A::IPW > Dd::IPW ? A::IPW : Dd::IPW) > (Cc::IPW > E::IPW ? Cc::IPW : E::IPW)
+                                  ? (A::IPW > Dd::IPW ? A::IPW : Dd::IPW)
+                                  : (Cc::IPW > E::IPW ? Cc::IPW : E::IPW);
+};
+
+template <class C, int MAXKV>
 __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a) {
+  typedef Phases<C> PS;
+  typedef typename PS::A PA;
+  typedef typename PS::Cc PC;
+  typedef typename PS::Dd PD;
+  typedef typename PS::E PE;
+  constexpr int D = C::D, HS = C::HS, H = C::H, HID = C::HID, SPLIT = C::SPLIT, MAXI = PS::MAXI;
+  constexpr int XS = C::SH * SEG;                                   // floats of the input row buffer
+  constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;     // floats of the staged exchange words
+  constexpr int CPWMAX = PA::CPW > PD::CPW ? PA::CPW : PD::CPW;
+  constexpr int PART = 32 * (HS + 4) > CPWMAX * NW ? 32 * (HS + 4) : CPWMAX * NW;
+
   extern __shared__ float lds[];
+  float* xs = lds;            // [XS]
+  float* attp = xs + XS;      // [ATTP]
+  float* part = attp + ATTP;  // [PART]
+  float* qkv_s = part + PART; // [3*HS]
+  float* hw = qkv_s + 3 * HS; // [H*SPLIT] per-slice merge weights
 
-  // LDS carve-up (floats): xs [a.xs_floats] | att partials [a.attp_floats] | part | qkv_s | own residual
-  float* xs = lds;
-  float* attp = xs + a.xs_floats;
-  float* part = attp + a.attp_floats;
-  float* qkv_s = part + a.part_floats;
-
-  const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
-  const int d = a.d, hs = a.hs, H = a.H, hid = 4 * a.d;
+  const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
   if (tid == 0) sh.bail = 0;
-  for (int e = tid; e < a.xs_floats; e += NT) xs[e] = 0.f;
+  for (int e = tid; e < XS; e += NT) xs[e] = 0.f;
   __syncthreads();
 
-  // attention role: head and slice of the positions
-  const bool att_role = wg < H * a.split;
-  const int ah = wg / a.split, as = wg - ah * a.split;
-  // attention threads: 32 key groups (tid >> 4) of 16 lanes (tid & 15), hs = 64
+  // items of this workgroup per phase (fewer than ITEMS only when N is not a multiple of G*CPW)
+  auto items_of = [&](int N, int CPW, int S) {
+    int n = N - wg * CPW;
+    n = n > CPW ? CPW : (n < 0 ? 0 : n);
+    return n * S;
+  };
+  const int nitA = items_of(PA::N, PA::CPW, PA::S), nitC = items_of(PC::N, PC::CPW, PC::S);
+  const int nitD = items_of(PD::N, PD::CPW, PD::S), nitE = items_of(PE::N, PE::CPW, PE::S);
 
-  // columns this workgroup finishes in the d-wide phases (C and E share geometry N = d)
-  const int colC0 = wg * a.gC.cpw;
-  int ncolC = d - colC0;
-  ncolC = ncolC > a.gC.cpw ? a.gC.cpw : (ncolC < 0 ? 0 : ncolC);
+  // attention role: head and slice of the positions; threads form 32 key groups
+  // (tid >> 4) of 16 lanes (tid & 15)
+  const bool att_role = wg < H * SPLIT;
+  const int ah = wg / SPLIT, as = wg - ah * SPLIT;
 
-  WSet<MAXI> set0, set1;
+  const LayerParamOffsets po = layer_param_offsets(D);
+  WSet<MAXI> ws;
+  float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
   int tok = a.tok[0];
 
-  const LayerParamOffsets po = layer_param_offsets(d);
-  load_items<MAXI>(set0, a.slabs, a.gA, d, a.lparams + po.bA, wg, wave, lane);
+  load_items<PA, MAXI>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+  load_ln<D, MAXI>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b);
 
   for (int step = 0; step < a.nsteps; ++step) {
     const int pos = a.pos0 + step;
+    TRACE(0);
     // ---- embedding: every workgroup builds the row itself (instructions.js:795-821) ----
-    for (int e = tid; e < d; e += NT) xs[e] = a.wte[(size_t)tok * d + e] + a.wpe[(size_t)pos * d + e];
+    for (int e = tid; e < D; e += NT) xs[e] = a.wte[(size_t)tok * D + e] + a.wpe[(size_t)pos * D + e];
     __syncthreads();
 
     // slice of positions 0..pos for the attention role
     const int nkeys = pos + 1;
-    const int chunk = (nkeys + a.split - 1) / a.split;
+    const int chunk = (nkeys + SPLIT - 1) / SPLIT;
     const int c0 = as * chunk;
     int c1 = c0 + chunk;
     c1 = c1 > nkeys ? nkeys : c1;
+    const bool has_new = pos >= c0 && pos < c1;  // this slice holds the new position
+    const int nkv = c1 > c0 ? (c1 - c0 + 31) / 32 : 0;  // key batches of this slice
+
+    float own_r = 0.f;  // residual stream value of the column this thread finishes in the d-wide phases
 
     for (int li = 0; li < a.L; ++li) {
       const float4* slab = a.slabs + (size_t)li * a.slab_stride;
       const float* lp = a.lparams + (size_t)li * po.stride;
-      float* Kc = a.kv + ((size_t)(li * 2 + 0) * H + ah) * a.ctx * hs;
-      float* Vc = a.kv + ((size_t)(li * 2 + 1) * H + ah) * a.ctx * hs;
+      float* Kc = a.kv + ((size_t)(li * 2 + 0) * H + ah) * a.ctx * HS;
+      float* Vc = a.kv + ((size_t)(li * 2 + 1) * H + ah) * a.ctx * HS;
 
-      // ================= phase A: LN1 + QKV =================
-      if (li > 0) {
-        if (!poll_words(a.bufR2, d, ep, xs, a.err)) {}
-        __syncthreads();
-        if (sh.bail) return;
-      }
-      const float own_r = tid < ncolC ? xs[colC0 + tid] : 0.f;  // residual of the columns finished in phase C
-      layernorm_lds(xs, d, lp + po.ln1g, lp + po.ln1b);
-      // request what is needed two phases ahead: proj weights and this layer's cached keys/values
-      load_items<MAXI>(set1, slab + a.slab_offC, a.gC, d, lp + po.bC, wg, wave, lane);
-      float4 kreg[MAXKV], vreg[MAXKV];
-      if (att_role) {
-        const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
-#pragma unroll
-        for (int i = 0; i < MAXKV; ++i) {
-          const int j = c0 + g16 + 32 * i;
-          float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
-          if (j < c1 && j < pos) {
-            const u64* kp = reinterpret_cast<const u64*>(Kc + (size_t)j * hs + sub * 4);
-            const u64* vp = reinterpret_cast<const u64*>(Vc + (size_t)j * hs + sub * 4);
-            const u64 k0 = ld_word(kp), k1 = ld_word(kp + 1), v0 = ld_word(vp), v1 = ld_word(vp + 1);
-            kk = make_float4(__uint_as_float((unsigned)k0), __uint_as_float((unsigned)(k0 >> 32)),
-                             __uint_as_float((unsigned)k1), __uint_as_float((unsigned)(k1 >> 32)));
-            vv = make_float4(__uint_as_float((unsigned)v0), __uint_as_float((unsigned)(v0 >> 32)),
-                             __uint_as_float((unsigned)v1), __uint_as_float((unsigned)(v1 >> 32)));
-          }
-          kreg[i] = kk;
-          vreg[i] = vv;
-        }
-      }
-      gemv_items<MAXI>(set0, xs, part, a.gA, wg, wave, lane);
-      __syncthreads();
-      ++ep;
+      // ======================= c_attn: LN1 + QKV =======================
       {
-        const int col0 = wg * a.gA.cpw;
-        int ncols = 3 * d - col0;
-        ncols = ncols > a.gA.cpw ? a.gA.cpw : ncols;
-        if (tid < ncols) publish(a.bufQKV + col0 + tid, column_sum(part, a.gA, tid) + set0.bias, ep);
+        constexpr int PH = PH_QKV;
+        if (li > 0) {
+          poll_words<D>(a.bufR2, ep, xs, a.err);
+          __syncthreads();
+          if (sh.bail) return;
+        }
+        wait_loads();
+        TRACE(1 + li * 8 + PH);
+        own_r = (tid < PC::CPW && wg * PC::CPW + tid < D) ? xs[wg * PC::CPW + tid] : 0.f;
+        layernorm_lds<D, MAXI>(xs, ws, lane);
+        TRACE5(1);
+        gemv_items<PA, MAXI>(ws, xs, part, nitA, wave, lane);
+        TRACE5(2);
+        __syncthreads();
+        ++ep;
+        if (tid < PA::CPW && wg * PA::CPW + tid < PA::N)
+          publish(a.bufQKV + wg * PA::CPW + tid, column_sum<PA>(part, tid) + ws.bias, ep);
+        TRACE5(4);
+        load_items<PC, MAXI>(ws, slab + a.slab_offC, lp + po.bC, nitC, wg, wave, lane);
+        TRACE5(5);
+        if (att_role) {
+          // this layer's cached keys and values of the slice
+          const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
+#pragma unroll
+          for (int i = 0; i < MAXKV; ++i) {
+            const int j = c0 + g16 + 32 * i;
+            float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
+            if (i < nkv && j < c1 && j < pos) {
+              const u64* kp = reinterpret_cast<const u64*>(Kc + (size_t)j * HS + sub * 4);
+              const u64* vp = reinterpret_cast<const u64*>(Vc + (size_t)j * HS + sub * 4);
+              const u64 k0 = ld_word(kp), k1 = ld_word(kp + 1), v0 = ld_word(vp), v1 = ld_word(vp + 1);
+              kk = make_float4(__uint_as_float((unsigned)k0), __uint_as_float((unsigned)(k0 >> 32)),
+                               __uint_as_float((unsigned)k1), __uint_as_float((unsigned)(k1 >> 32)));
+              vv = make_float4(__uint_as_float((unsigned)v0), __uint_as_float((unsigned)(v0 >> 32)),
+                               __uint_as_float((unsigned)v1), __uint_as_float((unsigned)(v1 >> 32)));
+            }
+            kreg[i] = kk;
+            vreg[i] = vv;
+          }
+        }
+        TRACE5(6);
       }
 
-      // ================= phase B: attention slice =================
-      // fc weights go where the QKV weights were
-      load_items<MAXI>(set0, slab + a.slab_offD, a.gD, d, lp + po.bD, wg, wave, lane);
-      ++ep;
+      // ======================= attention slice (role workgroups) =======================
+      ++ep;  // epoch of the attention outputs
       if (att_role) {
-        // q, k, v of this head for the new token
         {
-          unsigned pending = tid < 3 * hs ? 1u : 0u;
+          unsigned pending = tid < 3 * HS ? 1u : 0u;
           unsigned spins = 0;
-          const int which = tid / hs, e = tid - which * hs;
-          const u64* src = a.bufQKV + which * d + ah * hs + e;
+          const int which = tid / HS, e = tid - which * HS;
+          const u64* src = a.bufQKV + which * D + ah * HS + e;
           while (pending) {
             const u64 pk = ld_word(src);
             if ((unsigned)(pk >> 32) == ep - 1) {
@@ -351,11 +473,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         __syncthreads();
         if (sh.bail) return;
+        wait_loads();
+        TRACE(1 + li * 8 + 5);
         // the slice that holds the new position appends it to the cache and uses it from LDS
-        const bool has_new = pos >= c0 && pos < c1;
         if (has_new && tid < 32) {
-          const float* src = qkv_s + (tid < 16 ? hs : 2 * hs) + (tid & 15) * 4;
-          float* dstp = (tid < 16 ? Kc : Vc) + (size_t)pos * hs + (tid & 15) * 4;
+          const float* src = qkv_s + (tid < 16 ? HS : 2 * HS) + (tid & 15) * 4;
+          float* dstp = (tid < 16 ? Kc : Vc) + (size_t)pos * HS + (tid & 15) * 4;
           u64* dp = reinterpret_cast<u64*>(dstp);
           st_word(dp, ((u64)__float_as_uint(src[1]) << 32) | __float_as_uint(src[0]));
           st_word(dp + 1, ((u64)__float_as_uint(src[3]) << 32) | __float_as_uint(src[2]));
@@ -366,150 +489,190 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         float m = -INFINITY;
 #pragma unroll
         for (int i = 0; i < MAXKV; ++i) {
-          const int j = c0 + g16 + 32 * i;
-          if (j == pos && has_new) {
-            kreg[i] = *reinterpret_cast<const float4*>(qkv_s + hs + sub * 4);
-            vreg[i] = *reinterpret_cast<const float4*>(qkv_s + 2 * hs + sub * 4);
+          sc[i] = -INFINITY;
+          if (i < nkv) {
+            const int j = c0 + g16 + 32 * i;
+            if (j == pos && has_new) {
+              kreg[i] = *reinterpret_cast<const float4*>(qkv_s + HS + sub * 4);
+              vreg[i] = *reinterpret_cast<const float4*>(qkv_s + 2 * HS + sub * 4);
+            }
+            const float p = row16_sum((qv.x * kreg[i].x + qv.y * kreg[i].y) + (qv.z * kreg[i].z + qv.w * kreg[i].w));
+            sc[i] = j < c1 ? p * a.scale : -INFINITY;
+            m = fmaxf(m, sc[i]);
           }
-          float p = (qv.x * kreg[i].x + qv.y * kreg[i].y) + (qv.z * kreg[i].z + qv.w * kreg[i].w);
-          p += __shfl_xor(p, 8);
-          p += __shfl_xor(p, 4);
-          p += __shfl_xor(p, 2);
-          p += __shfl_xor(p, 1);
-          sc[i] = j < c1 ? p * a.scale : -INFINITY;
-          m = fmaxf(m, sc[i]);
         }
-        m = fmaxf(m, __shfl_xor(m, 16));
-        m = fmaxf(m, __shfl_xor(m, 32));
-        if (lane == 0) sh.red[wave] = m;
+        if (sub == 0) sh.red[g16] = m;
         __syncthreads();
 #pragma unroll
-        for (int v = 0; v < NW; ++v) m = fmaxf(m, sh.red[v]);
+        for (int v = 0; v < 32; ++v) m = fmaxf(m, sh.red[v]);
         float l = 0.f;
         float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
         if (m > -INFINITY) {
 #pragma unroll
           for (int i = 0; i < MAXKV; ++i) {
-            const float p = sc[i] > -INFINITY ? expf(sc[i] - m) : 0.f;
-            l += p;
-            o.x += p * vreg[i].x; o.y += p * vreg[i].y; o.z += p * vreg[i].z; o.w += p * vreg[i].w;
-          }
-        }
-        // combine the 32 key groups: 4 per wave by shuffles, then 8 waves through LDS
-        o.x += __shfl_xor(o.x, 16); o.y += __shfl_xor(o.y, 16); o.z += __shfl_xor(o.z, 16); o.w += __shfl_xor(o.w, 16);
-        o.x += __shfl_xor(o.x, 32); o.y += __shfl_xor(o.y, 32); o.z += __shfl_xor(o.z, 32); o.w += __shfl_xor(o.w, 32);
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
-        __syncthreads();  // sh.red reads above are done
-        if (lane < 16) *reinterpret_cast<float4*>(part + wave * (hs + 4) + lane * 4) = o;
-        if (lane == 0) part[wave * (hs + 4) + hs] = l;
-        __syncthreads();
-        if (tid < hs + 2) {
-          float v = 0.f;
-          if (tid < hs) {
-#pragma unroll
-            for (int w8 = 0; w8 < NW; ++w8) v += part[w8 * (hs + 4) + tid];
-          } else if (tid == hs) {
-            v = m;
-          } else {
-#pragma unroll
-            for (int w8 = 0; w8 < NW; ++w8) v += part[w8 * (hs + 4) + hs];
-          }
-          publish(a.bufATT + (size_t)wg * (hs + 2) + tid, v, ep);
-        }
-      }
-
-      // ================= phase C: merge slices, projection, residual =================
-      if (!poll_words(a.bufATT, H * a.split * (hs + 2), ep, attp, a.err)) {}
-      __syncthreads();
-      if (sh.bail) return;
-      for (int e = tid; e < d; e += NT) {
-        const int h = e / hs, c = e - h * hs;
-        const float* ph = attp + (size_t)h * a.split * (hs + 2);
-        float M = -INFINITY;
-        for (int s2 = 0; s2 < a.split; ++s2) M = fmaxf(M, ph[s2 * (hs + 2) + hs]);
-        float Lsum = 0.f, val = 0.f;
-        for (int s2 = 0; s2 < a.split; ++s2) {
-          const float ms = ph[s2 * (hs + 2) + hs];
-          const float wgt = ms > -INFINITY ? expf(ms - M) : 0.f;
-          Lsum += ph[s2 * (hs + 2) + hs + 1] * wgt;
-          val += ph[s2 * (hs + 2) + c] * wgt;
-        }
-        xs[e] = val / Lsum;
-      }
-      __syncthreads();
-      // fc2 weights go where the projection weights are, after they have been used:
-      gemv_items<MAXI>(set1, xs, part, a.gC, wg, wave, lane);
-      __syncthreads();
-      ++ep;
-      float r1 = 0.f;
-      if (tid < ncolC) {
-        r1 = column_sum(part, a.gC, tid) + set1.bias + own_r;
-        publish(a.bufR1 + colC0 + tid, r1, ep);
-      }
-      load_items<MAXI>(set1, slab + a.slab_offE, a.gE, hid, lp + po.bE, wg, wave, lane);
-
-      // ================= phase D: LN2 + fc + GELU =================
-      if (!poll_words(a.bufR1, d, ep, xs, a.err)) {}
-      __syncthreads();
-      if (sh.bail) return;
-      layernorm_lds(xs, d, lp + po.ln2g, lp + po.ln2b);
-      gemv_items<MAXI>(set0, xs, part, a.gD, wg, wave, lane);
-      __syncthreads();
-      ++ep;
-      {
-        const int col0 = wg * a.gD.cpw;
-        int ncols = hid - col0;
-        ncols = ncols > a.gD.cpw ? a.gD.cpw : ncols;
-        if (tid < ncols) publish(a.bufH + col0 + tid, gelu_ref(column_sum(part, a.gD, tid) + set0.bias), ep);
-      }
-      // next layer's QKV weights (or nothing after the last layer)
-      if (li + 1 < a.L) load_items<MAXI>(set0, slab + a.slab_stride, a.gA, d, lp + po.stride + po.bA, wg, wave, lane);
-      else if (step + 1 < a.nsteps) load_items<MAXI>(set0, a.slabs, a.gA, d, a.lparams + po.bA, wg, wave, lane);
-
-      // ================= phase E: fc2 + residual =================
-      if (!poll_words(a.bufH, hid, ep, xs, a.err)) {}
-      __syncthreads();
-      if (sh.bail) return;
-      gemv_items<MAXI>(set1, xs, part, a.gE, wg, wave, lane);
-      __syncthreads();
-      ++ep;
-      if (tid < ncolC) publish(a.bufR2 + colC0 + tid, column_sum(part, a.gE, tid) + set1.bias + r1, ep);
-      // xs beyond d must be zero again for the d-wide phases that follow
-      for (int e = d + tid; e < a.xs_floats; e += NT) xs[e] = 0.f;
-      __syncthreads();
-    }
-
-    // ================= final LayerNorm + vocabulary projection =================
-    if (!poll_words(a.bufR2, d, ep, xs, a.err)) {}
-    __syncthreads();
-    if (sh.bail) return;
-    layernorm_lds(xs, d, a.lnf_g, a.lnf_b);
-    {
-      const int v0 = wg * a.rows_per_wg;
-      int v1 = v0 + a.rows_per_wg;
-      v1 = v1 > a.V ? a.V : v1;
-      float best = -INFINITY;
-      int besti = 0x7fffffff;
-      const int S = a.gA.S;
-      for (int vb = v0 + wave * 4; vb < v1; vb += NW * 4) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int s2 = 0; s2 < S; ++s2) {
-          const int k = s2 * SEG + lane * 4;
-          if (k < d) {
-            const float4 x = *reinterpret_cast<const float4*>(xs + k);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              if (vb + r < v1) {
-                const float4 w = *reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * d + k);
-                acc[r] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
-              }
+            if (i < nkv) {
+              const float p = sc[i] > -INFINITY ? expf(sc[i] - m) : 0.f;
+              l += p;
+              o.x += p * vreg[i].x; o.y += p * vreg[i].y; o.z += p * vreg[i].z; o.w += p * vreg[i].w;
             }
           }
         }
+        // the 32 key groups combine through LDS
+        *reinterpret_cast<float4*>(part + g16 * (HS + 4) + sub * 4) = o;
+        if (sub == 0) part[g16 * (HS + 4) + HS] = l;
+        __syncthreads();
+        if (tid < HS + 2) {
+          float v = 0.f;
+          if (tid == HS) {
+            v = m;
+          } else {
+            const int c = tid < HS ? tid : HS;
+#pragma unroll 8
+            for (int g2 = 0; g2 < 32; ++g2) v += part[g2 * (HS + 4) + c];
+          }
+          publish(a.bufATT + (size_t)wg * (HS + 2) + tid, v, ep);
+        }
+      }
+
+      // ======================= attention c_proj: merge slices, project, residual =======================
+      {
+        constexpr int PH = PH_PROJ;
+        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err);
+        __syncthreads();
+        if (sh.bail) return;
+        wait_loads();
+        TRACE(1 + li * 8 + PH);
+        // per (head, slice): weight exp(m_s - M) / L of the slice's unnormalised output
+        if (tid < H) {
+          const float* phd = attp + tid * SPLIT * (HS + 2);
+          float M = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float s = wave_sum(acc[r]);
+          for (int s2 = 0; s2 < SPLIT; ++s2) M = fmaxf(M, phd[s2 * (HS + 2) + HS]);
+          float wv[SPLIT];
+          float Lsum = 0.f;
+#pragma unroll
+          for (int s2 = 0; s2 < SPLIT; ++s2) {
+            const float ms = phd[s2 * (HS + 2) + HS];
+            wv[s2] = ms > -INFINITY ? expf(ms - M) : 0.f;
+            Lsum += phd[s2 * (HS + 2) + HS + 1] * wv[s2];
+          }
+#pragma unroll
+          for (int s2 = 0; s2 < SPLIT; ++s2) hw[tid * SPLIT + s2] = wv[s2] / Lsum;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < (D + NT - 1) / NT; ++k) {
+          const int e = tid + k * NT;
+          if (k * NT + NT <= D || e < D) {
+            const int h = e / HS, c = e - h * HS;
+            const float* phd = attp + h * SPLIT * (HS + 2) + c;
+            float val = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < SPLIT; ++s2) val += phd[s2 * (HS + 2)] * hw[h * SPLIT + s2];
+            xs[e] = val;
+          }
+        }
+        __syncthreads();
+        TRACE5(1);
+        gemv_items<PC, MAXI>(ws, xs, part, nitC, wave, lane);
+        TRACE5(2);
+        __syncthreads();
+        ++ep;
+        if (tid < PC::CPW && wg * PC::CPW + tid < D) {
+          own_r += column_sum<PC>(part, tid) + ws.bias;  // model.js:159
+          publish(a.bufR1 + wg * PC::CPW + tid, own_r, ep);
+        }
+        TRACE5(4);
+        load_items<PD, MAXI>(ws, slab + a.slab_offD, lp + po.bD, nitD, wg, wave, lane);
+        load_ln<D, MAXI>(ws, lp + po.ln2g, lp + po.ln2b);
+        TRACE5(5);
+      }
+
+      // ======================= c_fc: LN2 + fc + GELU =======================
+      {
+        constexpr int PH = PH_FC;
+        poll_words<D>(a.bufR1, ep, xs, a.err);
+        __syncthreads();
+        if (sh.bail) return;
+        wait_loads();
+        TRACE(1 + li * 8 + PH);
+        layernorm_lds<D, MAXI>(xs, ws, lane);
+        TRACE5(1);
+        gemv_items<PD, MAXI>(ws, xs, part, nitD, wave, lane);
+        TRACE5(2);
+        __syncthreads();
+        ++ep;
+        if (tid < PD::CPW && wg * PD::CPW + tid < HID)
+          publish(a.bufH + wg * PD::CPW + tid, gelu_ref(column_sum<PD>(part, tid) + ws.bias), ep);  // model.js:188
+        TRACE5(4);
+        load_items<PE, MAXI>(ws, slab + a.slab_offE, lp + po.bE, nitE, wg, wave, lane);
+        TRACE5(5);
+      }
+
+      // ======================= mlp c_proj: fc2 + residual =======================
+      {
+        constexpr int PH = PH_FC2;
+        poll_words<HID>(a.bufH, ep, xs, a.err);
+        __syncthreads();
+        if (sh.bail) return;
+        wait_loads();
+        TRACE(1 + li * 8 + PH);
+        gemv_items<PE, MAXI>(ws, xs, part, nitE, wave, lane);
+        TRACE5(2);
+        __syncthreads();
+        ++ep;
+        if (tid < PC::CPW && wg * PC::CPW + tid < D)
+          publish(a.bufR2 + wg * PC::CPW + tid, own_r + column_sum<PE>(part, tid) + ws.bias, ep);  // model.js:205
+        TRACE5(4);
+        // next layer's c_attn share, or the first layer's for the next step
+        if (li + 1 < a.L) {
+          load_items<PA, MAXI>(ws, slab + a.slab_stride, lp + po.stride + po.bA, nitA, wg, wave, lane);
+          load_ln<D, MAXI>(ws, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
+        } else {
+          load_ln<D, MAXI>(ws, a.lnf_g, a.lnf_b);
+        }
+        TRACE5(5);
+        // xs beyond D must be zero again for the D-wide phases that follow
+        for (int e = D + tid; e < XS; e += NT) xs[e] = 0.f;
+        __syncthreads();
+      }
+    }
+
+    // ======================= final LayerNorm + vocabulary projection =======================
+    poll_words<D>(a.bufR2, ep, xs, a.err);
+    __syncthreads();
+    if (sh.bail) return;
+    wait_loads();
+    TRACE(1 + a.L * 8);
+    layernorm_lds<D, MAXI>(xs, ws, lane);
+    {
+      constexpr int S = C::SD, R = 4;  // rows of wte in flight per wave
+      const int lane = opaque(tid & 63);
+      const int v0 = wg * a.rows_per_wg;
+      int v1 = v0 + a.rows_per_wg;
+      v1 = v1 > a.V ? a.V : v1;
+      float4 xv[S];
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2) xv[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
+      float best = -INFINITY;
+      int besti = 0x7fffffff;
+      for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
+        float4 w[R][S];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int s2 = 0; s2 < S; ++s2) {
+            w[r][s2] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (vb + r < v1 && (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D))
+              w[r][s2] = ld_stream(reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * D + s2 * SEG + lane * 4));
+          }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s2 = 0; s2 < S; ++s2)
+            acc += (w[r][s2].x * xv[s2].x + w[r][s2].y * xv[s2].y) + (w[r][s2].z * xv[s2].z + w[r][s2].w * xv[s2].w);
+          const float s = wave_sum(acc);
           if (vb + r < v1) {
             if (lane == 0) a.logits[vb + r] = s;
             if (s > best || besti == 0x7fffffff) {
@@ -540,14 +703,20 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         publish(a.bufAM + 2 * wg + 1, __int_as_float(bi), ep);
       }
     }
-    // ================= arg-max over the workgroups, finished by everyone =================
-    if (!poll_words(a.bufAM, 2 * a.G, ep, attp, a.err)) {}
+    TRACE(2 + a.L * 8);
+    if (step + 1 < a.nsteps) {
+      load_items<PA, MAXI>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+      load_ln<D, MAXI>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b);
+    }
+    // ======================= arg-max over the workgroups, finished by everyone =======================
+    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err);
     __syncthreads();
     if (sh.bail) return;
+    TRACE(3 + a.L * 8);
     {
       float b = -INFINITY;
       int bi = 0x7fffffff;
-      for (int w2 = lane; w2 < a.G; w2 += 64) {
+      for (int w2 = lane; w2 < C::G; w2 += 64) {
         const float ov = attp[2 * w2];
         const int oi = __float_as_int(attp[2 * w2 + 1]);
         if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > b || (ov == b && oi < bi))) {
@@ -588,61 +757,66 @@ __global__ void build_slab_kernel(const float* __restrict__ W, int ldw, int K, i
   slab[idx] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-template <int MAXI, int MAXKV>
-hipError_t launch_t(const PersistentArgs& a, size_t lds_bytes, hipStream_t s) {
-  auto kern = decode_persistent_kernel<MAXI, MAXKV>;
-  static size_t allowed = 0;  // dynamic LDS size already enabled for this instantiation
-  if (lds_bytes > allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return e;
-    allowed = lds_bytes;
-  }
-  kern<<<a.G, NT, lds_bytes, s>>>(a);
-  return hipGetLastError();
-}
-
-}  // namespace
-
-PhaseGeom make_geom(int N, int K, int G) {
-  PhaseGeom g;
-  g.N = N;
-  g.cpw = (N + G - 1) / G;
-  g.S = (K + SEG - 1) / SEG;
-  g.ipw = (g.cpw * g.S + NW - 1) / NW;
-  return g;
-}
-
-size_t slab_float4s(const PhaseGeom& g, int G) { return (size_t)G * g.cpw * g.S * 64; }
-
-hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, int G, float4* slab, hipStream_t s) {
-  const size_t total = slab_float4s(g, G);
-  build_slab_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(W, ldw, K, g.N, g.cpw, g.S, total, slab);
-  return hipGetLastError();
-}
-
-int persistent_max_items(const PersistentArgs& a) {
-  int m = a.gA.ipw;
-  m = a.gC.ipw > m ? a.gC.ipw : m;
-  m = a.gD.ipw > m ? a.gD.ipw : m;
-  m = a.gE.ipw > m ? a.gE.ipw : m;
-  return m;
-}
-
-size_t persistent_lds_bytes(const PersistentArgs& a) {
-  const size_t need = sizeof(float) * ((size_t)a.xs_floats + a.attp_floats + a.part_floats + 3 * a.hs + 16);
+template <class C>
+size_t lds_bytes_of() {
+  typedef Phases<C> PS;
+  constexpr int XS = C::SH * SEG;
+  constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;
+  constexpr int CPWMAX = PS::A::CPW > PS::Dd::CPW ? PS::A::CPW : PS::Dd::CPW;
+  constexpr int PART = 32 * (C::HS + 4) > CPWMAX * NW ? 32 * (C::HS + 4) : CPWMAX * NW;
+  const size_t need = sizeof(float) * (size_t)(XS + ATTP + PART + 3 * C::HS + C::H * C::SPLIT + 16);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
   const size_t one_per_cu = 84 * 1024;
   return need > one_per_cu ? need : one_per_cu;
 }
 
+template <class C>
+hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
+  auto kern = decode_persistent_kernel<C, PD_MAXKV>;
+  const size_t lds_bytes = lds_bytes_of<C>();
+  static bool enabled = false;  // dynamic LDS size already raised for this instantiation
+  if (!enabled) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    enabled = true;
+  }
+  kern<<<PD_GRID, NT, lds_bytes, s>>>(a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+PhaseGeom make_geom(int N, int K) {
+  PhaseGeom g;
+  g.N = N;
+  g.cpw = (N + PD_GRID - 1) / PD_GRID;
+  g.S = (K + SEG - 1) / SEG;
+  g.ipw = (g.cpw * g.S + NW - 1) / NW;
+  return g;
+}
+
+size_t slab_float4s(const PhaseGeom& g) { return (size_t)PD_GRID * g.cpw * g.S * 64; }
+
+hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4* slab, hipStream_t s) {
+  const size_t total = slab_float4s(g);
+  build_slab_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(W, ldw, K, g.N, g.cpw, g.S, total, slab);
+  return hipGetLastError();
+}
+
+bool persistent_supports(int d, int n_head, int n_ctx) {
+  if (((n_ctx + PD_SPLIT - 1) / PD_SPLIT + 31) / 32 > PD_MAXKV) return false;
+  return (d == 384 && n_head == 6) || (d == 768 && n_head == 12) || (d == 1024 && n_head == 16) ||
+         (d == 1280 && n_head == 20);
+}
+
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
-  const int mi = persistent_max_items(a);
-  const size_t lds = persistent_lds_bytes(a);
-  const int kv_per_thread = ((a.ctx + a.split - 1) / a.split + 31) / 32;
-  if (kv_per_thread > 8) return hipErrorInvalidValue;
-  if (mi <= 4) return launch_t<4, 8>(a, lds, s);
-  if (mi <= 8) return launch_t<8, 8>(a, lds, s);
-  if (mi <= 16) return launch_t<16, 8>(a, lds, s);
+  if (!persistent_supports(a.d, a.H, a.ctx)) return hipErrorInvalidValue;
+  switch (a.d) {
+    case 384: return launch_t<Shape<384, 6>>(a, s);
+    case 768: return launch_t<Shape<768, 12>>(a, s);
+    case 1024: return launch_t<Shape<1024, 16>>(a, s);
+    case 1280: return launch_t<Shape<1280, 20>>(a, s);
+  }
   return hipErrorInvalidValue;
 }
 

@@ -4,6 +4,7 @@
 // from a device-resident KV cache).
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <unordered_map>
@@ -184,36 +185,24 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 // m->persist_ok false (and the per-block path in charge) for shapes it does not cover.
 static int setup_persistent(Model* m) {
   m->persist_ok = false;
-  const int d = m->d, hid = 4 * d, G = 256, split = 4;
+  const int d = m->d, hid = 4 * d, G = PD_GRID, split = PD_SPLIT;
   if (m->p.weight_dtype != 0 || m->hs != 64) return WGPT_OK;
   if (rt().compute_units < G) return WGPT_OK;
+  if (!persistent_supports(d, m->H, m->ctx)) return WGPT_OK;
   PersistentArgs& a = m->pa;
   a = PersistentArgs{};
-  a.L = m->L; a.H = m->H; a.d = d; a.hs = m->hs; a.ctx = m->ctx; a.V = m->V;
-  a.G = G; a.split = split;
+  a.L = m->L; a.H = m->H; a.d = d; a.ctx = m->ctx; a.V = m->V;
   a.scale = (float)(1.0 / std::sqrt((double)m->hs));
-  a.gA = make_geom(3 * d, d, G);
-  a.gC = make_geom(d, d, G);
-  a.gD = make_geom(hid, d, G);
-  a.gE = make_geom(d, hid, G);
+  const PhaseGeom gA = make_geom(3 * d, d), gC = make_geom(d, d), gD = make_geom(hid, d), gE = make_geom(d, hid);
   a.rows_per_wg = (m->V + G - 1) / G;
   const int attw = m->H * split * (m->hs + 2);
-  if (persistent_max_items(a) > 16 || hid > 8192 || attw > 8192 || m->H * split > G) return WGPT_OK;
-  if (((m->ctx + split - 1) / split + 31) / 32 > 8) return WGPT_OK;
-  a.xs_floats = a.gE.S * 256;
-  a.attp_floats = attw > 2 * G ? attw : 2 * G;
-  int pf = 8 * (m->hs + 4);
-  const int cpw_max = a.gD.cpw > a.gA.cpw ? a.gD.cpw : a.gA.cpw;
-  if (cpw_max * 8 > pf) pf = cpw_max * 8;
-  a.part_floats = pf;
-  if (persistent_lds_bytes(a) > 150 * 1024) return WGPT_OK;
 
   int rc;
   // all slabs in one allocation, all small per-layer parameters in another
-  a.slab_offC = slab_float4s(a.gA, G);
-  a.slab_offD = a.slab_offC + slab_float4s(a.gC, G);
-  a.slab_offE = a.slab_offD + slab_float4s(a.gD, G);
-  a.slab_stride = a.slab_offE + slab_float4s(a.gE, G);
+  a.slab_offC = slab_float4s(gA);
+  a.slab_offD = a.slab_offC + slab_float4s(gC);
+  a.slab_offE = a.slab_offD + slab_float4s(gD);
+  a.slab_stride = a.slab_offE + slab_float4s(gE);
   float4* slabs;
   if ((rc = dev_alloc(m, a.slab_stride * (size_t)m->L * sizeof(float4), (void**)&slabs))) return rc;
   const LayerParamOffsets po = layer_param_offsets(d);
@@ -222,10 +211,10 @@ static int setup_persistent(Model* m) {
   for (int i = 0; i < m->L; ++i) {
     const LayerW& l = m->layers[i];
     float4* sl = slabs + (size_t)i * a.slab_stride;
-    LAUNCH(build_slab(l.attn.w, 3 * d, d, a.gA, G, sl, rt().stream));
-    LAUNCH(build_slab(l.proj.w, d, d, a.gC, G, sl + a.slab_offC, rt().stream));
-    LAUNCH(build_slab(l.fc.w, hid, d, a.gD, G, sl + a.slab_offD, rt().stream));
-    LAUNCH(build_slab(l.fc2.w, d, hid, a.gE, G, sl + a.slab_offE, rt().stream));
+    LAUNCH(build_slab(l.attn.w, 3 * d, d, gA, sl, rt().stream));
+    LAUNCH(build_slab(l.proj.w, d, d, gC, sl + a.slab_offC, rt().stream));
+    LAUNCH(build_slab(l.fc.w, hid, d, gD, sl + a.slab_offD, rt().stream));
+    LAUNCH(build_slab(l.fc2.w, d, hid, gE, sl + a.slab_offE, rt().stream));
     float* lp = lparams + (size_t)i * po.stride;
     const struct { int off; const float* src; int n; } parts[8] = {
         {po.bA, l.attn_b, 3 * d}, {po.bC, l.proj_b, d}, {po.bD, l.fc_b, hid}, {po.bE, l.fc2_b, d},
@@ -254,6 +243,12 @@ static int setup_persistent(Model* m) {
   a.tok = m->tok_dev;
   a.out_tok = m->out_tok_dev;
   a.err = m->perr;
+  a.trace = nullptr;
+#ifdef WGPT_TRACE
+  // Profiling builds: per-workgroup clock samples of the last step of each launch.
+  if ((rc = dev_alloc(m, sizeof(unsigned long long) * 512 * G, (void**)&a.trace))) return rc;
+  WGPT_HIP(hipMemsetAsync(a.trace, 0, sizeof(unsigned long long) * 512 * G, rt().stream));
+#endif
   m->epoch = 0;
   m->persist_ok = true;
   return WGPT_OK;
@@ -266,7 +261,7 @@ static int decode_persistent(Model* m, int steps) {
   const unsigned per_step = persistent_epochs_per_step(m->L);
   if (m->epoch > 0xffffffffu - per_step * (unsigned)steps - 8u) {
     // epoch counter about to wrap: start over from clean exchange buffers
-    const size_t words = (size_t)(a.bufAM + 2 * a.G - a.bufQKV);
+    const size_t words = (size_t)(a.bufAM + 2 * PD_GRID - a.bufQKV);
     WGPT_HIP(hipMemsetAsync(a.bufQKV, 0, words * sizeof(unsigned long long), rt().stream));
     m->epoch = 0;
   }
@@ -280,6 +275,16 @@ static int decode_persistent(Model* m, int steps) {
 
 // After the stream has drained: did a bounded wait of the persistent kernel expire?
 static int check_persistent(Model* m) {
+#ifdef WGPT_TRACE
+  if (const char* path = getenv("WGPT_TRACE_FILE")) {
+    std::vector<unsigned long long> h(512 * (size_t)PD_GRID);
+    WGPT_HIP(hipMemcpy(h.data(), m->pa.trace, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    if (FILE* f = fopen(path, "wb")) {
+      fwrite(h.data(), sizeof(unsigned long long), h.size(), f);
+      fclose(f);
+    }
+  }
+#endif
   int herr = 0;
   WGPT_HIP(hipMemcpy(&herr, m->perr, sizeof(int), hipMemcpyDeviceToHost));
   if (herr != 0) {
