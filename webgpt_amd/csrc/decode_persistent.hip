@@ -27,18 +27,21 @@
 #include "decode_persistent.h"
 
 #include <cstdio>
+#include <type_traits>
 
 namespace wgpt {
 
 namespace {
 
 typedef unsigned long long u64;
+#ifndef WGPT_DBG_SKIP_W
+#define WGPT_DBG_SKIP_W 0
+#endif
 
 constexpr int NT = PD_THREADS;       // threads per workgroup
 constexpr int NW = NT / 64;          // waves per workgroup
 constexpr int SEG = 256;             // contraction elements per item (64 lanes x float4)
 constexpr int NPMAX = 8;             // a poll round covers up to NPMAX*NT words
-constexpr int LNMAX = 4;             // LayerNorm parameters held per thread: d <= LNMAX*NT
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 
 __device__ __forceinline__ u64 ld_word(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -144,7 +147,6 @@ struct Shape {
   static constexpr int SH = (HID + SEG - 1) / SEG;    // segments of a HID-long contraction
   static constexpr int ATTW = H * SPLIT * (HS + 2);   // words of the attention exchange buffer
   static_assert(HS == 64, "the attention phase is laid out for head size 64");
-  static_assert(D <= LNMAX * NT, "LayerNorm parameter registers cover d <= 2048");
 };
 
 // One linear phase: N outputs from a K-long input.
@@ -155,6 +157,7 @@ struct Phase {
   static constexpr int S = (K + SEG - 1) / SEG;            // segments per column
   static constexpr int ITEMS = CPW * S;                    // items per workgroup
   static constexpr int IPW = (ITEMS + NW - 1) / NW;        // items per wave
+  static constexpr bool RAGGED = CPW * PD_GRID != N;       // some workgroups finish fewer than CPW columns
 };
 
 // Polls N {value, epoch} words until all carry `epoch`, storing the values to dst
@@ -194,70 +197,129 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
 
 // Registers of one linear phase: this wave's share of the weight slab (MAXI float4
 // per lane), the bias of the column this thread finishes, and the LayerNorm
-// parameters of the elements this thread normalises (phases with a LayerNorm).
-template <int MAXI>
+// parameters of the lane's elements of every segment (phases with a LayerNorm).
+template <int MAXI, int SD>
 struct WSet {
   float4 w[MAXI];
   float bias;
-  float g[LNMAX], b[LNMAX];
+  float4 g[SD], b[SD];
 };
+
+// Calls f(std::integral_constant<int, wave>) so that everything derived from the
+// wave index is a compile-time constant inside f (one copy of the code per wave).
+template <class F>
+__device__ __forceinline__ void for_wave(int wave, F f) {
+  switch (wave) {
+    case 0: f(std::integral_constant<int, 0>()); break;
+    case 1: f(std::integral_constant<int, 1>()); break;
+    case 2: f(std::integral_constant<int, 2>()); break;
+    case 3: f(std::integral_constant<int, 3>()); break;
+    case 4: f(std::integral_constant<int, 4>()); break;
+    case 5: f(std::integral_constant<int, 5>()); break;
+    case 6: f(std::integral_constant<int, 6>()); break;
+    default: f(std::integral_constant<int, 7>()); break;
+  }
+}
 
 // Requests the slab share of this wave: items [wave*IPW, wave*IPW + IPW) of the
 // workgroup's `nitems`; item j is 64 consecutive float4 (column j / S, segment j % S).
-template <class P, int MAXI>
-__device__ __forceinline__ void load_items(WSet<MAXI>& ws, const float4* __restrict__ slab, const float* __restrict__ bias,
+template <class P, class WS>
+__device__ __forceinline__ void load_items(WS& ws, const float4* __restrict__ slab, const float* __restrict__ bias,
                                            int nitems, int wg, int wave, int lane) {
-  static_assert(P::IPW <= MAXI, "register set too small");
-  const float4* base = slab + ((size_t)wg * P::ITEMS + (size_t)wave * P::IPW) * 64 + opaque(lane);
-  const int j0 = opaque_s(wave) * P::IPW;
+  const float4* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
+  for_wave(wave, [&](auto W) {
+    constexpr int J0 = decltype(W)::value * P::IPW;
 #pragma unroll
-  for (int i = 0; i < P::IPW; ++i) {
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (j0 + i < nitems) v = ld_stream(base + i * 64);
-    ws.w[i] = v;
-  }
+    for (int i = 0; i < P::IPW; ++i) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (J0 + i < P::ITEMS) {
+        if (!P::RAGGED || J0 + i < nitems) v = ld_stream(wgbase + (J0 + i) * 64);
+      }
+      ws.w[i] = v;
+    }
+  });
   const int t = opaque(threadIdx.x);
   ws.bias = (t < P::CPW && wg * P::CPW + t < P::N) ? bias[wg * P::CPW + t] : 0.f;
 }
 
-// Requests the LayerNorm parameters of elements tid, tid+NT, ... of a D-wide row.
-template <int D, int MAXI>
-__device__ __forceinline__ void load_ln(WSet<MAXI>& ws, const float* __restrict__ gamma, const float* __restrict__ beta) {
-  const int t = threadIdx.x;
+// Requests the LayerNorm parameters of this lane's four elements of every segment.
+template <int D, class WS>
+__device__ __forceinline__ void load_ln(WS& ws, const float* __restrict__ gamma, const float* __restrict__ beta, int lane) {
+  constexpr int S = (D + SEG - 1) / SEG;
+  const int k0 = opaque(lane) * 4;
 #pragma unroll
-  for (int k = 0; k < (D + NT - 1) / NT; ++k) {
-    const int e = t + k * NT;
-    ws.g[k] = e < D ? gamma[e] : 0.f;
-    ws.b[k] = e < D ? beta[e] : 0.f;
+  for (int s2 = 0; s2 < S; ++s2) {
+    const bool in = s2 * SEG + SEG <= D || s2 * SEG + k0 < D;
+    ws.g[s2] = in ? *reinterpret_cast<const float4*>(gamma + s2 * SEG + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+    ws.b[s2] = in ? *reinterpret_cast<const float4*>(beta + s2 * SEG + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
 }
 
-// Dot products of this wave's items with the input vector xs (LDS, zero padded up
-// to S*SEG). Per (column, wave) partial sums go to part[col*NW + wave].
-template <class P, int MAXI>
-__device__ __forceinline__ void gemv_items(const WSet<MAXI>& ws, const float* xs, float* part, int nitems, int wave, int lane) {
-  lane = opaque(lane);
-  const int j0 = opaque_s(wave) * P::IPW;
-  int col = j0 / P::S;
-  int seg = j0 - col * P::S;
-  float acc = 0.f;
+// This wave's share of the matrix-vector product. The input row is read from xs
+// (LDS, zero padded up to S*SEG) into registers; with LNORM it is first normalised
+// there (instructions.js:451-550: biased variance about the mean, eps inside the
+// sqrt; the quotient (x - mean) / stdev is formed as (x - mean) * (1 / stdev)).
+// Every wave derives the two statistics itself, so no barrier is needed. Per
+// (column, wave) partial sums go to part[col*NW + wave].
+template <class P, bool LNORM, class WS>
+__device__ __forceinline__ void gemv_items(const WS& ws, const float* xs, float* part, int nitems, int wave, int lane) {
+  constexpr int S = P::S;
+  const float* xl = xs + opaque(lane) * 4;
+  for_wave(wave, [&](auto W) {
+    constexpr int WV = decltype(W)::value;
+    constexpr int J0 = WV * P::IPW;
+    // segments this wave needs: all of them for the statistics, else those of its items
+    float4 xr[S];
 #pragma unroll
-  for (int i = 0; i < P::IPW; ++i) {
-    if (j0 + i < nitems) {
-      const float4 x = *reinterpret_cast<const float4*>(xs + seg * SEG + lane * 4);
-      const float4 w = ws.w[i];
-      acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
-      if (seg == P::S - 1 || i == P::IPW - 1 || j0 + i == nitems - 1) {
-        const float r = wave_sum(acc);
-        if (lane == 0) part[col * NW + wave] = r;
-        acc = 0.f;
+    for (int s2 = 0; s2 < S; ++s2) {
+      bool used = LNORM;
+      for (int i = 0; i < P::IPW; ++i)
+        if (J0 + i < P::ITEMS && (J0 + i) % S == s2) used = true;
+      xr[s2] = used ? *reinterpret_cast<const float4*>(xl + s2 * SEG) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (LNORM) {
+      float sum = 0.f;
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2) sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
+      const float mean = wave_sum(sum) / (float)P::K;
+      float q = 0.f;
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2) {
+        // lanes beyond K hold zeros that must not count as (0 - mean)^2
+        const bool in = s2 * SEG + SEG <= P::K || s2 * SEG + lane * 4 < P::K;
+        xr[s2].x -= mean; xr[s2].y -= mean; xr[s2].z -= mean; xr[s2].w -= mean;
+        const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
+        q += in ? qq : 0.f;
       }
-      if (++seg == P::S) {
-        seg = 0;
-        ++col;
+      const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)P::K + 1e-5f);
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2) {
+        xr[s2].x = ws.g[s2].x * (xr[s2].x * rstd) + ws.b[s2].x;
+        xr[s2].y = ws.g[s2].y * (xr[s2].y * rstd) + ws.b[s2].y;
+        xr[s2].z = ws.g[s2].z * (xr[s2].z * rstd) + ws.b[s2].z;
+        xr[s2].w = ws.g[s2].w * (xr[s2].w * rstd) + ws.b[s2].w;
       }
     }
-  }
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < P::IPW; ++i) {
+      constexpr int dummy = 0;
+      (void)dummy;
+      if (J0 + i < P::ITEMS) {
+        if (!P::RAGGED || J0 + i < nitems) {
+          const int seg = (J0 + i) % S, col = (J0 + i) / S;
+          const float4 x = xr[seg];
+          const float4 w = ws.w[i];
+          acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+          if (seg == S - 1 || i == P::IPW - 1 || J0 + i == P::ITEMS - 1) {
+            const float r = wave_sum(acc);
+            if (lane == 0) part[col * NW + WV] = r;
+            acc = 0.f;
+          }
+        }
+      }
+    }
+  });
 }
 
 // Sum of the per-wave partials of local column c, in ascending wave order.
@@ -269,40 +331,6 @@ __device__ __forceinline__ float column_sum(const float* part, int c) {
   float s = 0.f;
   for (int v = v0; v <= v1; ++v) s += part[c * NW + v];
   return s;
-}
-
-// LayerNorm of xs[0..D) in place (instructions.js:451-550 semantics: biased variance
-// about the mean, eps inside the sqrt, true division). Every wave derives the two
-// statistics itself from LDS, so only the write-back needs barriers. xs is zero
-// beyond D up to S*SEG.
-template <int D, int MAXI>
-__device__ __forceinline__ void layernorm_lds(float* xs, const WSet<MAXI>& ws, int lane) {
-  constexpr int S = (D + SEG - 1) / SEG;
-  float4 v[S];
-  float s = 0.f;
-#pragma unroll
-  for (int s2 = 0; s2 < S; ++s2) {
-    v[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
-    s += (v[s2].x + v[s2].y) + (v[s2].z + v[s2].w);
-  }
-  const float mean = wave_sum(s) / (float)D;
-  float q = 0.f;
-#pragma unroll
-  for (int s2 = 0; s2 < S; ++s2) {
-    if (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D) {
-      const float a0 = v[s2].x - mean, a1 = v[s2].y - mean, a2 = v[s2].z - mean, a3 = v[s2].w - mean;
-      q += (a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3);
-    }
-  }
-  const float stdev = sqrtf(wave_sum(q) / (float)D + 1e-5f);
-  __syncthreads();  // every wave has read xs
-  const int t = opaque(threadIdx.x);
-#pragma unroll
-  for (int k = 0; k < (D + NT - 1) / NT; ++k) {
-    const int e = t + k * NT;
-    if (k * NT + NT <= D || e < D) xs[e] = ws.g[k] * ((xs[e] - mean) / stdev) + ws.b[k];
-  }
-  __syncthreads();
 }
 
 #ifdef WGPT_TRACE
@@ -374,13 +402,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   const int ah = wg / SPLIT, as = wg - ah * SPLIT;
 
   const LayerParamOffsets po = layer_param_offsets(D);
-  WSet<MAXI> ws;
+  WSet<MAXI, C::SD> ws;
   float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
   int tok = a.tok[0];
 
-  load_items<PA, MAXI>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
-  load_ln<D, MAXI>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b);
+  load_items<PA>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+  load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
 
   for (int step = 0; step < a.nsteps; ++step) {
     const int pos = a.pos0 + step;
@@ -417,16 +445,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         own_r = (tid < PC::CPW && wg * PC::CPW + tid < D) ? xs[wg * PC::CPW + tid] : 0.f;
-        layernorm_lds<D, MAXI>(xs, ws, lane);
-        TRACE5(1);
-        gemv_items<PA, MAXI>(ws, xs, part, nitA, wave, lane);
+        gemv_items<PA, true>(ws, xs, part, nitA, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
         if (tid < PA::CPW && wg * PA::CPW + tid < PA::N)
           publish(a.bufQKV + wg * PA::CPW + tid, column_sum<PA>(part, tid) + ws.bias, ep);
         TRACE5(4);
-        load_items<PC, MAXI>(ws, slab + a.slab_offC, lp + po.bC, nitC, wg, wave, lane);
+        load_items<PC>(ws, slab + a.slab_offC, lp + po.bC, nitC, wg, wave, lane);
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -574,7 +600,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         __syncthreads();
         TRACE5(1);
-        gemv_items<PC, MAXI>(ws, xs, part, nitC, wave, lane);
+        gemv_items<PC, false>(ws, xs, part, nitC, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
@@ -583,8 +609,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           publish(a.bufR1 + wg * PC::CPW + tid, own_r, ep);
         }
         TRACE5(4);
-        load_items<PD, MAXI>(ws, slab + a.slab_offD, lp + po.bD, nitD, wg, wave, lane);
-        load_ln<D, MAXI>(ws, lp + po.ln2g, lp + po.ln2b);
+        load_items<PD>(ws, slab + a.slab_offD, lp + po.bD, nitD, wg, wave, lane);
+        load_ln<D>(ws, lp + po.ln2g, lp + po.ln2b, lane);
         TRACE5(5);
       }
 
@@ -596,16 +622,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        layernorm_lds<D, MAXI>(xs, ws, lane);
-        TRACE5(1);
-        gemv_items<PD, MAXI>(ws, xs, part, nitD, wave, lane);
+        gemv_items<PD, true>(ws, xs, part, nitD, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
         if (tid < PD::CPW && wg * PD::CPW + tid < HID)
           publish(a.bufH + wg * PD::CPW + tid, gelu_ref(column_sum<PD>(part, tid) + ws.bias), ep);  // model.js:188
         TRACE5(4);
-        load_items<PE, MAXI>(ws, slab + a.slab_offE, lp + po.bE, nitE, wg, wave, lane);
+        load_items<PE>(ws, slab + a.slab_offE, lp + po.bE, nitE, wg, wave, lane);
         TRACE5(5);
       }
 
@@ -617,7 +641,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        gemv_items<PE, MAXI>(ws, xs, part, nitE, wave, lane);
+        gemv_items<PE, false>(ws, xs, part, nitE, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
@@ -626,10 +650,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE5(4);
         // next layer's c_attn share, or the first layer's for the next step
         if (li + 1 < a.L) {
-          load_items<PA, MAXI>(ws, slab + a.slab_stride, lp + po.stride + po.bA, nitA, wg, wave, lane);
-          load_ln<D, MAXI>(ws, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
+          load_items<PA>(ws, slab + a.slab_stride, lp + po.stride + po.bA, nitA, wg, wave, lane);
+          load_ln<D>(ws, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b, lane);
         } else {
-          load_ln<D, MAXI>(ws, a.lnf_g, a.lnf_b);
+          load_ln<D>(ws, a.lnf_g, a.lnf_b, lane);
         }
         TRACE5(5);
         // xs beyond D must be zero again for the D-wide phases that follow
@@ -644,16 +668,39 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     if (sh.bail) return;
     wait_loads();
     TRACE(1 + a.L * 8);
-    layernorm_lds<D, MAXI>(xs, ws, lane);
     {
       constexpr int S = C::SD, R = 4;  // rows of wte in flight per wave
       const int lane = opaque(tid & 63);
       const int v0 = wg * a.rows_per_wg;
       int v1 = v0 + a.rows_per_wg;
       v1 = v1 > a.V ? a.V : v1;
+      // final LayerNorm of the row, in registers (each wave for itself)
       float4 xv[S];
+      {
+        float sum = 0.f;
 #pragma unroll
-      for (int s2 = 0; s2 < S; ++s2) xv[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
+        for (int s2 = 0; s2 < S; ++s2) {
+          xv[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
+          sum += (xv[s2].x + xv[s2].y) + (xv[s2].z + xv[s2].w);
+        }
+        const float mean = wave_sum(sum) / (float)D;
+        float q = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < S; ++s2) {
+          const bool in = s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D;
+          xv[s2].x -= mean; xv[s2].y -= mean; xv[s2].z -= mean; xv[s2].w -= mean;
+          const float qq = (xv[s2].x * xv[s2].x + xv[s2].y * xv[s2].y) + (xv[s2].z * xv[s2].z + xv[s2].w * xv[s2].w);
+          q += in ? qq : 0.f;
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)D + 1e-5f);
+#pragma unroll
+        for (int s2 = 0; s2 < S; ++s2) {
+          xv[s2].x = ws.g[s2].x * (xv[s2].x * rstd) + ws.b[s2].x;
+          xv[s2].y = ws.g[s2].y * (xv[s2].y * rstd) + ws.b[s2].y;
+          xv[s2].z = ws.g[s2].z * (xv[s2].z * rstd) + ws.b[s2].z;
+          xv[s2].w = ws.g[s2].w * (xv[s2].w * rstd) + ws.b[s2].w;
+        }
+      }
       float best = -INFINITY;
       int besti = 0x7fffffff;
       for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
@@ -705,8 +752,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
     TRACE(2 + a.L * 8);
     if (step + 1 < a.nsteps) {
-      load_items<PA, MAXI>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
-      load_ln<D, MAXI>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b);
+      load_items<PA>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+      load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
     poll_words<2 * C::G>(a.bufAM, ep, attp, a.err);
