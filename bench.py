@@ -106,6 +106,11 @@ def main():
         per_tok.append((time.perf_counter() - t0) * 1000.0)
         nxt = int(np.argmax(lg))
 
+    persistent = args.mode in (None, 1) and cfg["dtype"] == "f32"
+    kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
+                   else "per-block kernels (all launches of one token)")
+    # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)
+    traffic = 523.5e6 if (persistent and args.config == "gpt2-117m") else None
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
@@ -131,9 +136,12 @@ def main():
         "host_loop_ms_per_token": {"mean": round(float(np.mean(per_tok)), 4), "p50": round(float(np.median(per_tok)), 4),
                                    "note": "wgpt_decode per token incl. logits read-back over PCIe"} if per_tok else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "one decode token (all launches of the token)",
-                     "bytes_per_step": int(bytes_total / args.steps)},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "kernel": kernel_name,
+                     "bytes_per_step": int(bytes_total / args.steps),
+                     "note": "achieved = algorithmic bytes (weights + KV rows read) of the timed steps / HIP-event time of "
+                             "the launch(es) that ran them; traffic = measured HBM bytes of one step (rocprofv3 FETCH_SIZE + "
+                             "WRITE_SIZE, profiles/), null where no counter run exists for the configuration"},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt)

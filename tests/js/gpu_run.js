@@ -1,0 +1,40 @@
+// Runs the toy GPT through the JavaScript host on the GPU and prints results as JSON:
+// run() over a growing window (prefill once, then KV-cached decodes), the block-by-block
+// replay of the reference's pass list, generate() with top_k = 1 and the on-device greedy loop.
+"use strict";
+const w = require("../../webgpt_amd/js/index.js");
+const s = w.synth;
+
+async function main() {
+  const name = process.argv[2] || "toy";
+  const cfg = s.CONFIGS[name];
+  const fast = (seed, n, count, std) => w.native.synthNormal(seed, n, count, std);
+  const tensors = {};
+  for (const [n, a] of s.makeTensors(cfg, 1, fast)) tensors[n] = a;
+  const params = { n_layer: cfg.n_layer, n_head: cfg.n_head, n_embd: cfg.n_embd, n_ctx: cfg.n_ctx, vocab_size: cfg.vocab_size };
+  const gpt = new w.GPT(null, "char", { tensors, params });
+  await gpt.initialize();
+  const tokens = Array.from(s.tokens(1, "prompt", 24, cfg.vocab_size));
+  const out = { device: gpt.device.name, tokens };
+  let logits = await gpt.run(tokens.slice(0, 16));
+  out.logits16 = Array.from(logits);
+  for (let t = 16; t < 24; t++) logits = await gpt.run(tokens.slice(0, t + 1));
+  out.logits24 = Array.from(logits);
+  // the reference's pass list, block by block, whole window recomputed
+  const bw = gpt.loadBlockWeights(tensors);
+  out.blocks24 = Array.from(await gpt.runBlocks(tokens, bw));
+  // error path: the library's message becomes a thrown Error
+  try { await gpt.run([cfg.vocab_size]); out.badToken = null; } catch (e) { out.badToken = e.message; }
+  // generate() with top_k = 1, then the same continuation on the device
+  const gen = [];
+  for await (const id of gpt.generate(tokens.slice(0, 8), 10, 1, 1.0)) gen.push(id);
+  out.generated = gen;
+  const lg = await gpt.run(tokens.slice(0, 8));
+  let first = 0;
+  for (let i = 1; i < lg.length; i++) if (lg[i] > lg[first]) first = i;
+  out.greedy = [first].concat(Array.from(gpt.decodeGreedy(first, 9)));
+  gpt.unloadBuffers();
+  w.destroyOperations();
+  console.log(JSON.stringify(out));
+}
+main().catch((e) => { console.error(e); process.exit(1); });

@@ -1,0 +1,237 @@
+// GPT: the driver class of the reference's model.js over the HIP library.
+//
+// initialize() loads a weight directory (params_gpt.json + one little-endian f32
+// <tensor>_gpt.bin per tensor, model.js:270-488) or takes tensors from memory;
+// run(idx) resolves to the logits of the last token of the window idx
+// (model.js:104-268); generate() is the sampling loop of model.js:53-102.
+// run() is served from the device-resident KV cache whenever idx is the previous
+// window plus one token, else the whole window is recomputed (as the reference does
+// every token). runBlocks(idx) replays the reference's pass list block by block.
+"use strict";
+const fs = require("fs");
+const path = require("path");
+const { performance } = require("perf_hooks");
+const native = require("./native.js");
+const { Device, initTensor, runPasses } = require("./instructions.js");
+const G = require("./globals.js");
+
+class GPT {
+  constructor(folder, type, options = {}) {
+    this.folder = folder;
+    this.tokenizerType = type;
+    this.initialized = false;
+    this.device = undefined;
+    this.model = undefined;
+    this.tokenizer = options.tokenizer;
+    this.params = undefined;
+    this.minBufferOffset = 1;
+    this.defaultPrompt = undefined;
+    this.defaultTopK = undefined;
+    this.defaultTemperature = undefined;
+    this.defaultTokens = undefined;
+    this.externalBuffer = undefined;
+    this.unloadDeletionStack = [];
+    this._tensors = options.tensors;  // Map or object name -> TypedArray, instead of files
+    this._paramsIn = options.params;
+    this._flags = options.flags || 0;
+    this._history = [];
+    this.lastGpuMs = 0;
+  }
+
+  async initialize() {
+    if (this.initialized) return console.error("Model already initialized");
+    this.device = new Device(0);
+    G.initializeOperations(this.device);
+    [this.model, this.params] = await this.loadModel(this.folder);
+    if (this.tokenizerType == "bpe") {
+      this.defaultPrompt = `What is the answer to life, the universe, and everything?\n`;
+      this.defaultTopK = 3;
+      this.defaultTemperature = 1;
+      this.defaultTokens = 30;
+    } else {
+      this.defaultPrompt = `WILL:\nAh, how dare you challenge me?\nHave you forgotten I built WebGPT?\n`;
+      this.defaultTopK = 2;
+      this.defaultTemperature = 1;
+      this.defaultTokens = 80;
+    }
+    this.initialized = true;
+  }
+
+  async *generate(prompt, max_new_tokens, top_k, temperature) {
+    if (!this.initialized) {
+      console.error("Model not loaded yet");
+      return;
+    }
+    // prompt: a string when a tokenizer was given, else an array of token ids
+    let history = this.tokenizer ? this.tokenizer.encode(prompt) : Array.from(prompt);
+    const warmupRuns = 3;
+    let totalTime = 0;
+    for (let i = 0; i < max_new_tokens; i++) {
+      const idx_cond = history.slice(-this.params.n_ctx);
+      const startTime = performance.now();
+      const logits = await this.run(idx_cond);
+      const lapsedTime = performance.now() - startTime;
+      i >= warmupRuns && (totalTime += lapsedTime);
+      const { topKIndices, topKProbs } = G.selectTopK(logits, top_k);
+      const probs = G.cpuSoftmax(topKProbs, temperature);
+      const idx_next = topKIndices[G.sampleFromDistribution(probs)];
+      history = history.concat(idx_next);
+      yield this.tokenizer ? this.tokenizer.decode([idx_next]) : idx_next;
+    }
+    this.averageMs = totalTime / Math.max(1, max_new_tokens - warmupRuns);
+  }
+
+  async run(idx) {
+    const h = this._history;
+    const extends1 = h.length > 0 && idx.length === h.length + 1 && idx.length <= this.params.n_ctx && h.every((t, i) => t === idx[i]);
+    let logits;
+    if (extends1) {
+      logits = native.decode(this.model.handle, idx[idx.length - 1], this.params.vocab_size);
+      h.push(idx[idx.length - 1]);
+    } else {
+      logits = native.prefill(this.model.handle, Int32Array.from(idx), this.params.vocab_size);
+      this._history = Array.from(idx);
+    }
+    this.lastGpuMs = native.modelLastGpuMs(this.model.handle);
+    return logits;
+  }
+
+  // Greedy continuation entirely on the device: ids of `steps` tokens after `token`.
+  decodeGreedy(token, steps) {
+    const ids = native.decodeGreedy(this.model.handle, token, steps);
+    this._history = this._history.concat([token], Array.from(ids.slice(0, steps - 1)));
+    this.lastGpuMs = native.modelLastGpuMs(this.model.handle);
+    return ids;
+  }
+
+  // The reference's pass list (model.js:118-240) built block by block from separately
+  // uploaded weights and replayed through the per-block entry points.
+  async runBlocks(idx, weights) {
+    const { n_embd, n_head, head_size, n_layer, vocab_size, hidden_size, attention_scale } = this.params;
+    const seq_length = idx.length;
+    const passesAll = [];
+    let intermediateBuffer, residualBuffer;
+    const push = ({ passes, resultBuffer }) => {
+      passesAll.push(...passes);
+      return resultBuffer;
+    };
+    intermediateBuffer = residualBuffer = push(G.EmbedBlock.newInstance(idx, seq_length, n_embd, vocab_size, [weights.wte], weights.wpe, G.ResidualBlock));
+    for (let i = 0; i < n_layer; i++) {
+      const b = weights.layers[i];
+      intermediateBuffer = push(G.LayerNormBlock.newInstance(seq_length, n_embd, intermediateBuffer, b.normAttentionGammaBuffer, b.normAttentionBetaBuffer));
+      intermediateBuffer = push(G.AttentionBlock.newFusedInstance(seq_length, n_embd, attention_scale, n_head, head_size, intermediateBuffer,
+        b.qkvWeightArray[0], b.qkvBiasArray[0], b.qkvWeightArray[1], b.qkvBiasArray[1], b.qkvWeightArray[2], b.qkvBiasArray[2],
+        b.linearWeightsBuffer, b.linearBiasBuffer, G.FastMatMulBlock, G.SoftmaxBlock));
+      intermediateBuffer = residualBuffer = push(G.ResidualBlock.newInstance(seq_length, n_embd, intermediateBuffer, residualBuffer));
+      intermediateBuffer = push(G.LayerNormBlock.newInstance(seq_length, n_embd, intermediateBuffer, b.normLinearGammaBuffer, b.normLinearBetaBuffer));
+      intermediateBuffer = push(G.FastMatMulBlock.newInstance(seq_length, hidden_size, n_embd, intermediateBuffer, b.firstLayerWeightsBuffer, b.firstLayerBiasBuffer));
+      intermediateBuffer = push(G.GeluBlock.newInstance(seq_length, hidden_size, intermediateBuffer));
+      intermediateBuffer = push(G.FastMatMulBlock.newInstance(seq_length, n_embd, hidden_size, intermediateBuffer, b.secondLayerWeightsBuffer, b.secondLayerBiasBuffer));
+      intermediateBuffer = residualBuffer = push(G.ResidualBlock.newInstance(seq_length, n_embd, intermediateBuffer, residualBuffer));
+    }
+    if (this.externalBuffer) {
+      passesAll.push({ flag: "copy", src: intermediateBuffer, srcOffset: 0, dst: this.externalBuffer, dstOffset: 0, size: this.bufferSize(seq_length, n_embd) });
+    }
+    intermediateBuffer = push(G.LayerNormBlock.newInstance(seq_length, n_embd, intermediateBuffer, weights.normGammaBuffer, weights.normBetaBuffer));
+    const resultBuffer = push(G.DeEmbedBlock.newInstance(n_embd, vocab_size, vocab_size, seq_length, vocab_size, intermediateBuffer, [weights.wte]));
+    runPasses(passesAll);
+    const out = resultBuffer.download();
+    G.clearOperationCache();
+    return out;
+  }
+
+  // Uploads a {name: Float32Array} weight directory as separate buffers with the
+  // reference's load-time transforms (model.js:339-482), for runBlocks.
+  loadBlockWeights(tensors) {
+    const { n_embd: d, n_layer, n_ctx, vocab_size, hidden_size } = this.params;
+    const get = (n) => tensors[n];
+    const T = (data, dims) => this.initTensor(data, dims, ["storage"]);
+    const layers = [];
+    for (let i = 0; i < n_layer; i++) {
+      const p = `transformer.h.${i}.`;
+      // fetchAndSplitQKVWeightTensors: columns 0..d, d..2d, 2d..3d of c_attn [d, 3d]
+      const w = get(p + "attn.c_attn.weight"), b = get(p + "attn.c_attn.bias");
+      const split = [0, 1, 2].map((part) => {
+        const out = new Float32Array(d * d);
+        for (let k = 0; k < d; k++) out.set(w.subarray(k * 3 * d + part * d, k * 3 * d + (part + 1) * d), k * d);
+        return T(out, [d, d]);
+      });
+      layers.push({
+        normAttentionGammaBuffer: T(get(p + "ln_1.weight"), [d]), normAttentionBetaBuffer: T(get(p + "ln_1.bias"), [d]),
+        qkvWeightArray: split, qkvBiasArray: [0, 1, 2].map((part) => T(b.subarray(part * d, (part + 1) * d), [d])),
+        linearWeightsBuffer: T(get(p + "attn.c_proj.weight"), [d, d]), linearBiasBuffer: T(get(p + "attn.c_proj.bias"), [d]),
+        normLinearGammaBuffer: T(get(p + "ln_2.weight"), [d]), normLinearBetaBuffer: T(get(p + "ln_2.bias"), [d]),
+        firstLayerWeightsBuffer: T(get(p + "mlp.c_fc.weight"), [d, hidden_size]), firstLayerBiasBuffer: T(get(p + "mlp.c_fc.bias"), [hidden_size]),
+        secondLayerWeightsBuffer: T(get(p + "mlp.c_proj.weight"), [hidden_size, d]), secondLayerBiasBuffer: T(get(p + "mlp.c_proj.bias"), [d]),
+      });
+    }
+    return {
+      layers, wte: T(get("transformer.wte.weight"), [vocab_size, d]), wpe: T(get("transformer.wpe.weight"), [n_ctx, d]),
+      normGammaBuffer: T(get("transformer.ln_f.weight"), [d]), normBetaBuffer: T(get("transformer.ln_f.bias"), [d]),
+    };
+  }
+
+  async loadModel(folder) {
+    if (this.initialized) return console.error("Model already loaded");
+    const params = await this.loadParameters(folder);
+    const names = this._tensors ? Object.keys(this._tensors) : this.directoryNames(params);
+    const int8 = names.some((n) => n.endsWith(".weight.q"));
+    const handle = native.modelCreate(params.n_layer, params.n_head, params.n_embd, params.n_ctx, params.vocab_size, int8 ? 1 : 0, params.max_prefill || 0, this._flags);
+    for (const name of names) {
+      const data = this._tensors ? this._tensors[name] : this.fetchBin(path.join(folder, `${name}_gpt.bin`));
+      native.modelSetTensor(handle, name, data);
+    }
+    native.modelFinalize(handle);
+    return [{ handle }, params];
+  }
+
+  async loadParameters(weightsFolder) {
+    const params = this._paramsIn ? Object.assign({}, this._paramsIn) : JSON.parse(fs.readFileSync(path.join(weightsFolder, "params_gpt.json"), "utf8"));
+    // model.js:294-297
+    if (params.n_embd % 4 !== 0) throw new Error("Model load failed: n_embd must be divisible by 4.");
+    if (params.n_embd % params.n_head !== 0) throw new Error("Model load failed: n_embd must be divisible by n_head.");
+    if ((params.n_embd / params.n_head) % 4 !== 0) throw new Error("Model load failed: n_embd / n_head must be divisible by 4.");
+    // the vocabulary is never split here: one buffer, one launch
+    params.vocab_chunk_size = params.vocab_size;
+    params.vocab_chunk_instances = 1;
+    params.head_size = params.n_embd / params.n_head;
+    params.hidden_size = params.n_embd * 4;
+    params.attention_scale = 1 / Math.sqrt(params.n_embd / params.n_head);
+    params.bias = params.bias == undefined ? true : params.bias;
+    return params;
+  }
+
+  directoryNames(params) {
+    const names = ["transformer.wte.weight", "transformer.wpe.weight"];
+    for (let i = 0; i < params.n_layer; i++) {
+      for (const s of ["ln_1.weight", "ln_1.bias", "attn.c_attn.weight", "attn.c_attn.bias", "attn.c_proj.weight", "attn.c_proj.bias",
+        "ln_2.weight", "ln_2.bias", "mlp.c_fc.weight", "mlp.c_fc.bias", "mlp.c_proj.weight", "mlp.c_proj.bias"]) names.push(`transformer.h.${i}.${s}`);
+    }
+    return names.concat(["transformer.ln_f.weight", "transformer.ln_f.bias"]);
+  }
+
+  fetchBin(file) {
+    const b = fs.readFileSync(file);
+    return new Float32Array(b.buffer, b.byteOffset, b.byteLength / 4);
+  }
+
+  initTensor(data, dims, ops) {
+    const buffer = initTensor(data, dims);
+    this.unloadDeletionStack.push(buffer);
+    return buffer;
+  }
+
+  unloadBuffers() {
+    this.unloadDeletionStack.map((buffer) => buffer.destroy());
+    this.unloadDeletionStack = [];
+    if (this.model) native.modelDestroy(this.model.handle);
+    this.model = undefined;
+    this.initialized = false;
+  }
+
+  bufferSize(dimX, dimY = 1, dimZ = 1) {
+    return Math.ceil((dimX * dimY * dimZ * Float32Array.BYTES_PER_ELEMENT) / this.minBufferOffset) * this.minBufferOffset;
+  }
+}
+
+module.exports = { GPT };
