@@ -175,3 +175,26 @@ def test_persistent_decode_matches_per_block_decode_and_oracle(device, name, ste
         ids[mode] = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), min(steps, 24))]
     assert ids[0] == ids[1]
     gpt.unloadBuffers()
+
+
+@pytest.mark.parametrize("name", ["gpt2-345m", "gpt2-774m"])
+def test_larger_shapes_decode_against_oracle(device, name):
+    # the persistent decode kernel is instantiated per model width; check the other widths too
+    cfg = dict(synth.CONFIGS[name])
+    cfg["n_layer"] = 4          # same width/heads/vocab, fewer layers: keeps the oracle run short
+    gpt, tensors = load(cfg, seed=2, random_ln=True)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(6, "prompt", 14, cfg["vocab_size"])
+    got = gpt.prefill(tokens[:9])
+    want = ref.forward(p, w, tokens[:9])
+    assert close(got, want), worst(got, want)
+    out = {}
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        gpt.prefill(tokens[:9])
+        out[mode] = [gpt.decode(int(tokens[9 + i])) for i in range(5)]
+    want = ref.forward(p, w, tokens)
+    for mode in (0, 1):
+        assert close(out[mode][-1], want), (mode, worst(out[mode][-1], want))
+    assert greedy_ok(out[1][-1], want)
+    gpt.unloadBuffers()

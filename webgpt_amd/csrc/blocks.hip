@@ -57,7 +57,10 @@ static int matmul_dev(int M, int N, int K, const float* A, const float* W, const
     if (rc) return rc;
     e = launch_gemv_kn(M, N, K, A, K, W, N, bias, C, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   } else {
-    e = launch_gemm(M, N, K, A, K, W, N, bias, C, N, EPI_NONE, nullptr, rt().stream);
+    void* ws;
+    int rc = scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
+    if (rc) return rc;
+    e = launch_gemm(M, N, K, A, K, W, N, bias, C, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   }
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "matmul launch: %s", hipGetErrorString(e));
   return WGPT_OK;
@@ -121,7 +124,7 @@ int wgpt_matmul_bias_i8(int M, int N, int K, wgpt_buf A, wgpt_buf Wq, wgpt_buf s
     int rc = scratch(1, sizeof(float) * (size_t)K * N, &wf);
     if (rc) return rc;
     e = launch_dequant_i8(K, N, wq, N / 4, sc, (float*)wf, N, rt().stream);
-    if (e == hipSuccess) e = launch_gemm(M, N, K, a, K, (const float*)wf, N, b, c, N, EPI_NONE, nullptr, rt().stream);
+    if (e == hipSuccess) e = launch_gemm(M, N, K, a, K, (const float*)wf, N, b, c, N, EPI_NONE, nullptr, nullptr, rt().stream);
   }
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "int8 matmul launch: %s", hipGetErrorString(e));
   return WGPT_OK;

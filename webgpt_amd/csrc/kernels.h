@@ -22,9 +22,12 @@ size_t gemv_workspace_floats(int M, int N, int K);
 hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
                           float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
 
-// Same contraction for any M through the tiled GEMM kernels.
+// Same contraction for any M through the tiled GEMM kernels (matrix cores for M >= 16).
+// workspace (gemm_workspace_floats(M, N) floats, may be null) enables split-K for
+// shapes with too few output tiles to fill the GPU.
+size_t gemm_workspace_floats(int M, int N);
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
-                       float* C, int ldc, int epi, const float* resid, hipStream_t s);
+                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
 
 // int8 weight-only variants: Wq is [K, ldwq] words holding 4 columns each.
 hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,

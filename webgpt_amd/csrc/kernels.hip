@@ -257,6 +257,97 @@ __global__ __launch_bounds__(WG) void gemm_tile64(int M, int N, int K, const flo
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// FastMatMulBlock as a dense contraction on the matrix cores (prefill, M >= 16):
+// C = epi(A . W + bias). fp32 MFMA v_mfma_f32_32x32x2_f32: per instruction a wave
+// multiplies a 32x2 slice of A by a 2x32 slice of W into a 32x32 fp32 accumulator
+// (16 VGPRs per lane). Workgroup tile TM x 64 (TM = 64 or 128), four waves in a 2x2
+// arrangement, each owning (TM/2) x 32 of C; K advances in steps of 16 through LDS
+// with the next step's global loads held in registers while the current one is
+// multiplied. A is staged as [m][k] with a row stride of 17 floats (lanes of an
+// A-operand read hit distinct banks), W as [k][n].
+// Operand lane mapping of the instruction: lane l supplies A[row l%32][k l/32] and
+// W[k l/32][col l%32]; accumulator register r of lane l is
+// C[row (r/4)*8 + (l/32)*4 + r%4][col l%32].
+// ---------------------------------------------------------------------------
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// With kchunk < K (split-K) slice blockIdx.z covers k in [z*kchunk, (z+1)*kchunk) and
+// writes its raw partial sums to C + z*M*ldc (bias, epilogue: gemv_reduce afterwards).
+template <int TM>
+__global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
+                                                 const float* __restrict__ W, int ldw, const float* __restrict__ bias,
+                                                 float* C, int ldc, int epi, const float* resid) {
+  constexpr int BK = 16, TN = 64, AST = BK + 1;
+  constexpr int RB = TM / 64;  // 32-row blocks per wave
+  __shared__ float As[TM * AST];
+  __shared__ float Bs[BK * TN];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * 32;
+  // global -> register staging: A tile TM x 16 (float4 along k), W tile 16 x 64 (float4 along n)
+  const int arow = tid >> 2, akq = (tid & 3) * 4;
+  const int brow = tid >> 4, bnq = (tid & 15) * 4;
+  float4 ga[RB], gb;
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const int m = m0 + arow + r * 64;
+      ga[r] = (m < M && k0 + akq < K) ? ld4(A + (size_t)m * lda + k0 + akq) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    gb = (k0 + brow < K && n0 + bnq < N) ? ld4(W + (size_t)(k0 + brow) * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      float* d = As + (arow + r * 64) * AST + akq;
+      d[0] = ga[r].x; d[1] = ga[r].y; d[2] = ga[r].z; d[3] = ga[r].w;
+    }
+    st4(Bs + brow * TN + bnq, gb);
+  };
+  f32x16 acc[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
+
+  const int kbeg = blockIdx.z * kchunk;
+  const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
+  C += (size_t)blockIdx.z * M * ldc;
+  K = kend;
+  fetch(kbeg);
+  for (int k0 = kbeg; k0 < kend; k0 += BK) {
+    stage();
+    __syncthreads();
+    if (k0 + BK < kend) fetch(k0 + BK);
+    const float* ap = As + (wm + (lane & 31)) * AST + (lane >> 5);
+    const float* bp = Bs + (lane >> 5) * TN + wn + (lane & 31);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      const float b = bp[kk * TN];
+#pragma unroll
+      for (int r = 0; r < RB; ++r) acc[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[r * 32 * AST + kk], b, acc[r], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int n = n0 + wn + (lane & 31);
+  if (n >= N) return;
+  const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = m0 + wm + r * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+      if (m < M) {
+        float v = acc[r][i] + bv;
+        if (epi == EPI_GELU) v = gelu_ref(v);
+        else if (epi == EPI_RESIDUAL) v += resid[(size_t)m * ldc + n];
+        C[(size_t)m * ldc + n] = v;
+      }
+    }
+}
+
 // ResidualBlock, instructions.js:381-382
 __global__ __launch_bounds__(WG) void residual_kernel(size_t n4, const float* a, const float* b, float* out) {
   const size_t i = (size_t)blockIdx.x * WG + threadIdx.x;
@@ -527,10 +618,29 @@ hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const fl
   return hipGetLastError();
 }
 
+size_t gemm_workspace_floats(int M, int N) { return (size_t)8 * M * N; }
+
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
-                       float* C, int ldc, int epi, const float* resid, hipStream_t s) {
-  const dim3 grid(cdiv(N, 64), cdiv(M, 64));
-  gemm_tile64<<<grid, WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  if (M < 16) {
+    // too few rows for a matrix-core tile: scalar-FMA tile kernel
+    gemm_tile64<<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+  } else if ((size_t)cdiv(N, 64) * cdiv(M, 128) >= 512) {
+    gemm_mfma<128><<<dim3(cdiv(N, 64), cdiv(M, 128)), WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+  } else {
+    // few tiles: split K so that every compute unit gets work; partial sums are
+    // combined in ascending order by gemv_reduce (deterministic), bias last
+    const unsigned tiles = cdiv(N, 64) * cdiv(M, 64);
+    int S = 1;
+    while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
+    if (S == 1) {
+      gemm_mfma<64><<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+    } else {
+      const int kchunk = (int)cdiv(cdiv(K, S), 16) * 16;
+      gemm_mfma<64><<<dim3(cdiv(N, 64), cdiv(M, 64), S), WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
+      gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+    }
+  }
   return hipGetLastError();
 }
 

@@ -97,12 +97,12 @@ static int linear(Model* m, int M, int N, int K, const float* A, int lda, const 
       e = launch_gemv_kn_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
     } else {
       e = launch_dequant_i8(K, N, w.q, N / 4, w.s, m->dq, N, s);
-      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, s);
+      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s);
     }
   } else if (M <= GEMV_MAX_ROWS) {
     e = launch_gemv_kn(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
   } else {
-    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, s);
+    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
   }
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "linear layer launch: %s", hipGetErrorString(e));
   return WGPT_OK;
@@ -394,6 +394,8 @@ int wgpt_model_finalize(wgpt_model h) {
   size_t ws = gemv_workspace_floats(GEMV_MAX_ROWS, 4 * (int)d, (int)d);
   const size_t ws2 = gemv_workspace_floats(GEMV_MAX_ROWS, (int)d, 4 * (int)d);
   if (ws2 > ws) ws = ws2;
+  const size_t ws3 = gemm_workspace_floats((int)T, 4 * (int)d);  // split-K partial sums of the prefill GEMMs
+  if (ws3 > ws) ws = ws3;
   if ((rc = dev_alloc(m, ws * f, (void**)&m->part))) return rc;
   if (i8 && (rc = dev_alloc(m, d * 4 * d * f, (void**)&m->dq))) return rc;
   if ((m->p.flags & WGPT_FLAG_TAPS) && (rc = dev_alloc(m, (size_t)(2 + 6 * m->L) * T * d * f, (void**)&m->taps))) return rc;
