@@ -1,0 +1,78 @@
+"""BASELINE configurations at full size. The oracle is too slow to recompute every
+step here, so these runs are checked through size-independent properties:
+
+  - KV-cache invariance: the logits of the last decode step equal the logits of a
+    fresh prefill of the whole token history (causality makes them the same
+    quantity; the two paths share no kernel for attention or the linear layers);
+  - the greedy chain is self-consistent: every generated id is the arg-max of the
+    logits the model gives for the history before it (spot-checked by prefill);
+  - the oracle itself at a few positions where it finishes in seconds.
+"""
+import numpy as np
+import pytest
+
+from oracle import ref
+from webgpt_amd import synth
+from webgpt_amd.model import GPT
+
+from helpers import close, oracle_weights, worst
+
+pytestmark = pytest.mark.gpu
+
+
+def greedy_ok(got_logits, want_logits):
+    g, w = int(np.argmax(got_logits)), int(np.argmax(want_logits))
+    if g == w:
+        return True
+    top2 = np.sort(want_logits)[-2:]
+    return abs(float(top2[1] - top2[0])) <= 1e-5 + 1e-4 * abs(float(top2[1]))
+
+
+def run_config(name, prompt_len, steps, oracle_at=(), max_prefill=0):
+    cfg = dict(synth.CONFIGS[name])
+    tensors = dict(synth.make_tensors(cfg, 1))
+    params = synth.model_params(cfg)
+    params["max_prefill"] = max_prefill
+    gpt = GPT(None, "bpe", tensors=tensors, params=params)
+    gpt.initialize()
+    prompt = [int(t) for t in synth.make_prompt(cfg, 1, prompt_len)]
+    logits = gpt.prefill(prompt)
+    first = int(np.argmax(logits))
+    ids, last = gpt.decode_greedy(first, steps, want_logits=True)
+    history = prompt + [first] + [int(t) for t in ids]
+    # last logits belong to the window history[:-1]
+    again = gpt.prefill(history[:-1])
+    assert close(last, again), worst(last, again)
+    assert greedy_ok(again, last) and int(np.argmax(last)) == history[-1]
+    # spot-check the chain in the middle
+    for cut in (prompt_len + steps // 3, prompt_len + 2 * steps // 3):
+        lg = gpt.prefill(history[:cut])
+        best = int(np.argmax(lg))
+        gap = float(lg[best] - lg[history[cut]])
+        assert best == history[cut] or gap <= 1e-5 + 1e-4 * abs(float(lg[best])), (cut, best, history[cut], gap)
+    for T in oracle_at:
+        want = ref.forward(synth.model_params(cfg), oracle_weights(tensors, cfg), np.array(history[:T], np.int32))
+        got = gpt.prefill(history[:T])
+        assert close(got, want), (T, worst(got, want))
+        assert greedy_ok(got, want)
+    gpt.unloadBuffers()
+
+
+def test_toy_full():
+    run_config("toy", 64, 128, oracle_at=(64, 192))
+
+
+def test_gpt2_117m_full():
+    run_config("gpt2-117m", 128, 256, oracle_at=(160,))
+
+
+def test_gpt2_345m_full():
+    run_config("gpt2-345m", 512, 511)          # fills the context of 1024 exactly
+
+
+def test_gpt2_774m_to_full_context():
+    run_config("gpt2-774m", 64, 959)           # decode up to the last position of the context
+
+
+def test_gpt2_1p5b_int8_full():
+    run_config("gpt2-1.5b-int8", 128, 64)
