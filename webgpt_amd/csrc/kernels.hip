@@ -517,6 +517,105 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   }
 }
 
+
+// Prefill attention for head size 64 with K and V tiled through LDS: one workgroup
+// per (head, block of 16 query rows). Keys are visited in tiles of 64: the K and V
+// rows of the tile are staged in LDS once and shared by the 16 queries (the
+// per-query kernel above re-reads every row from L2 for every query). Thread
+// (q = tid/16, c = tid%16): scores of query q for keys c, c+16, c+32, c+48 of the
+// tile (q row in registers, K rows from LDS), running softmax over tiles, then the
+// four output columns 4c..4c+3 of query q (weights through LDS, V rows from LDS).
+// Arithmetic as the reference up to re-association: scale after the dot
+// (instructions.js:1176), masked keys contribute nothing, exp(x - max) / sum.
+constexpr int ATQ = 16, ATK = 64, AHS = 64, AKS = AHS + 4;  // row stride of the staged tiles (bank spread)
+__device__ __forceinline__ float row16_allsum(float v) {
+  v += __shfl_xor(v, 8);
+  v += __shfl_xor(v, 4);
+  v += __shfl_xor(v, 2);
+  v += __shfl_xor(v, 1);
+  return v;
+}
+__device__ __forceinline__ float row16_allmax(float v) {
+  v = fmaxf(v, __shfl_xor(v, 8));
+  v = fmaxf(v, __shfl_xor(v, 4));
+  v = fmaxf(v, __shfl_xor(v, 2));
+  v = fmaxf(v, __shfl_xor(v, 1));
+  return v;
+}
+
+__global__ __launch_bounds__(WG) void attention_tile_kernel(int Tq, int pos0, float scale, const float* __restrict__ q, int ldq,
+                                                             const float* __restrict__ Kc, const float* __restrict__ Vc,
+                                                             size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
+  __shared__ float Ks[ATK * AKS];
+  __shared__ float Vs[ATK * AKS];
+  __shared__ float Ps[ATQ * ATK];
+  const int h = blockIdx.x, i0 = blockIdx.y * ATQ;
+  const int tid = threadIdx.x, qi = tid >> 4, c = tid & 15;
+  const int i = i0 + qi;                 // query row of this thread (may be >= Tq in the last block)
+  const int p = pos0 + i;                // its absolute position: keys 0..p are visible
+  const int pmax = pos0 + (i0 + ATQ - 1 < Tq - 1 ? i0 + ATQ - 1 : Tq - 1);
+  float4 qr[AHS / 4];
+#pragma unroll
+  for (int k = 0; k < AHS / 4; ++k)
+    qr[k] = i < Tq ? ld4(q + (size_t)i * ldq + h * AHS + 4 * k) : make_float4(0.f, 0.f, 0.f, 0.f);
+  const float* kbase = Kc + h * hstride;
+  const float* vbase = Vc + h * hstride;
+  float m = -INFINITY, l = 0.f;
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int j0 = 0; j0 <= pmax; j0 += ATK) {
+    __syncthreads();  // previous tile fully consumed
+    // stage the tile: 64 rows x 16 float4, 256 threads x 4
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = (tid >> 4) + 16 * r, col4 = tid & 15;
+      float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), vv = kv;
+      if (j0 + row <= pmax) {
+        kv = ld4(kbase + (size_t)(j0 + row) * ldkv + 4 * col4);
+        vv = ld4(vbase + (size_t)(j0 + row) * ldkv + 4 * col4);
+      }
+      st4(Ks + row * AKS + 4 * col4, kv);
+      st4(Vs + row * AKS + 4 * col4, vv);
+    }
+    __syncthreads();
+    // scores of keys c, c+16, c+32, c+48
+    float sc[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float* kr = Ks + (c + 16 * r) * AKS;
+      float a = 0.f;
+#pragma unroll
+      for (int k = 0; k < AHS / 4; ++k) {
+        const float4 kv = ld4(kr + 4 * k);
+        a += (qr[k].x * kv.x + qr[k].y * kv.y) + (qr[k].z * kv.z + qr[k].w * kv.w);
+      }
+      sc[r] = (j0 + c + 16 * r <= p) ? a * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[r]);
+    }
+    tmax = row16_allmax(tmax);
+    const float mnew = fmaxf(m, tmax);
+    // rows beyond Tq and fully masked tiles keep m = -inf: guard the exponentials
+    const float corr = mnew > -INFINITY ? expf(m - mnew) : 1.f;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float pr = sc[r] > -INFINITY ? expf(sc[r] - mnew) : 0.f;
+      Ps[qi * ATK + c + 16 * r] = pr;
+      psum += pr;
+    }
+    psum = row16_allsum(psum);
+    l = l * corr + psum;
+    m = mnew;
+    o.x *= corr; o.y *= corr; o.z *= corr; o.w *= corr;
+    __syncthreads();  // weights of the tile visible (only this query's 16 lanes wrote them, but waves differ in pace)
+    const float* pr = Ps + qi * ATK;
+    const float* vr = Vs + 4 * c;
+#pragma unroll 8
+    for (int j = 0; j < ATK; ++j) fma4(o, pr[j], ld4(vr + j * AKS));
+  }
+  if (i < Tq) st4(out + (size_t)i * ldo + h * AHS + 4 * c, make_float4(o.x / l, o.y / l, o.z / l, o.w / l));
+}
+
 __global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* __restrict__ src, int lds,
                                                         float* __restrict__ dst, int ldd) {
   const int r = blockIdx.y;
@@ -678,6 +777,11 @@ hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, flo
 
 hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
                             const float* Vc, size_t hstride, int ldkv, float* out, int ldo, hipStream_t s) {
+  // enough (head, query block) workgroups to fill the GPU; else one workgroup per query row
+  if (hs == AHS && Tq >= ATQ && H * cdiv(Tq, ATQ) >= 128) {
+    attention_tile_kernel<<<dim3(H, cdiv(Tq, ATQ)), WG, 0, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
+    return hipGetLastError();
+  }
   int lpk = 1;
   while (lpk * 4 < hs) lpk <<= 1;
   if (lpk > 64 || hs > 256 || (hs & 3)) return hipErrorInvalidValue;
