@@ -61,6 +61,7 @@ def main():
 
     from webgpt_amd import synth
     from webgpt_amd.model import GPT
+    from webgpt_amd._lib import WgptError
 
     cfg = dict(synth.CONFIGS[args.config])
     if cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
@@ -106,7 +107,13 @@ def main():
         per_tok.append((time.perf_counter() - t0) * 1000.0)
         nxt = int(np.argmax(lg))
 
-    persistent = args.mode in (None, 1) and cfg["dtype"] == "f32"
+    persistent = args.mode == 1
+    if args.mode is None:
+        try:  # the default mode is the persistent kernel wherever the library offers it for the shape
+            gpt.set_decode_mode(1)
+            persistent = True
+        except WgptError:
+            persistent = False
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
     # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)

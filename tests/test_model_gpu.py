@@ -198,3 +198,22 @@ def test_larger_shapes_decode_against_oracle(device, name):
         assert close(out[mode][-1], want), (mode, worst(out[mode][-1], want))
     assert greedy_ok(out[1][-1], want)
     gpt.unloadBuffers()
+
+
+def test_int8_persistent_decode_against_oracle(device):
+    # width of the 1.5B int8 configuration, two layers: persistent int8 decode vs per-block int8 decode vs oracle
+    cfg = dict(synth.CONFIGS["gpt2-1.5b-int8"])
+    cfg["n_layer"] = 2
+    gpt, tensors = load(cfg, seed=4, random_ln=True)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(6, "prompt", 13, cfg["vocab_size"])
+    out = {}
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        gpt.prefill(tokens[:8])
+        out[mode] = [gpt.decode(int(tokens[8 + i])) for i in range(5)]
+    want = ref.forward(p, w, tokens)
+    for mode in (0, 1):
+        assert close(out[mode][-1], want), (mode, worst(out[mode][-1], want))
+    assert greedy_ok(out[1][-1], want)
+    gpt.unloadBuffers()

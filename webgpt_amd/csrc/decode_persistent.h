@@ -22,15 +22,19 @@ struct PhaseGeom {
 };
 
 // Offsets (in floats) inside one layer's block of small parameters:
-// [c_attn bias 3d | attn c_proj bias d | c_fc bias 4d | mlp c_proj bias d | ln1 g,b | ln2 g,b].
+// [c_attn bias 3d | attn c_proj bias d | c_fc bias 4d | mlp c_proj bias d | ln1 g,b | ln2 g,b |
+//  int8 scales of the four matrices 3d, d, 4d, d].
 struct LayerParamOffsets {
-  int bA, bC, bD, bE, ln1g, ln1b, ln2g, ln2b, stride;
+  int bA, bC, bD, bE, ln1g, ln1b, ln2g, ln2b;
+  int sA, sC, sD, sE;  // per-column scales of the int8 variant (unused for fp32 weights)
+  int stride;
 };
 __host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
   LayerParamOffsets o;
   o.bA = 0; o.bC = 3 * d; o.bD = 4 * d; o.bE = 8 * d;
   o.ln1g = 9 * d; o.ln1b = 10 * d; o.ln2g = 11 * d; o.ln2b = 12 * d;
-  o.stride = 13 * d;
+  o.sA = 13 * d; o.sC = 16 * d; o.sD = 17 * d; o.sE = 21 * d;
+  o.stride = 22 * d;
   return o;
 }
 
@@ -38,11 +42,12 @@ struct PersistentArgs {
   int L, H, d, ctx, V;
   float scale;
   int rows_per_wg;  // vocabulary rows per workgroup
+  int weight_dtype;  // 0: fp32 items (float4 per lane), 1: int8 items (one word per lane)
   // slab-layout weights of all layers in one allocation: layer l starts at
-  // slabs + l*slab_stride; c_attn at 0, then attn c_proj, c_fc, mlp c_proj (float4 units)
-  const float4* slabs;
+  // slabs + l*slab_stride; c_attn at 0, then attn c_proj, c_fc, mlp c_proj (item-lane units)
+  const void* slabs;
   size_t slab_stride, slab_offC, slab_offD, slab_offE;
-  const float* lparams;  // [L][13d] small per-layer parameters (LayerParamOffsets)
+  const float* lparams;  // [L][22d] small per-layer parameters (LayerParamOffsets)
   const float *wte, *wpe, *lnf_g, *lnf_b;
   float* kv;  // [L][2][H][ctx][hs]
   // {value, epoch} exchange buffers
@@ -60,8 +65,10 @@ PhaseGeom make_geom(int N, int K);
 size_t slab_float4s(const PhaseGeom& g);
 // Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g.
 hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4* slab, hipStream_t s);
+// Same for int8 words Wq[K, ldwq] (4 columns per word): one word per item lane.
+hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g, int32_t* slab, hipStream_t s);
 // Model shapes the persistent kernel is instantiated for.
-bool persistent_supports(int d, int n_head, int n_ctx);
+bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype);
 // Epochs consumed by one decode step.
 inline unsigned persistent_epochs_per_step(int L) { return 5u * (unsigned)L + 1u; }
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s);

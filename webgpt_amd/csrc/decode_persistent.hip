@@ -139,9 +139,10 @@ __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70
 // constant, so the per-phase code is loads, FMAs and a few scalar compares. (A wave
 // retires only one instruction every few cycles; index arithmetic on the critical
 // path of a phase costs as much as the hop between phases.)
-template <int D_, int H_>
+template <int D_, int H_, bool I8_ = false>
 struct Shape {
   static constexpr int D = D_, H = H_, HS = D_ / H_, HID = 4 * D_;
+  static constexpr bool I8 = I8_;  // linear weights are int8 (4 contraction elements per 32-bit word) + per-column scale
   static constexpr int G = PD_GRID, SPLIT = PD_SPLIT;
   static constexpr int SD = (D + SEG - 1) / SEG;      // segments of a D-long contraction
   static constexpr int SH = (HID + SEG - 1) / SEG;    // segments of a HID-long contraction
@@ -198,12 +199,19 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
 // Registers of one linear phase: this wave's share of the weight slab (MAXI float4
 // per lane), the bias of the column this thread finishes, and the LayerNorm
 // parameters of the lane's elements of every segment (phases with a LayerNorm).
-template <int MAXI, int SD>
+template <int MAXI, int SD, bool I8>
 struct WSet {
-  float4 w[MAXI];
+  typename std::conditional<I8, int, float4>::type w[MAXI];  // an int8 item is one word per lane
   float bias;
+  float cscale;  // int8: scale[column] / 127 of the column this thread finishes
   float4 g[SD], b[SD];
 };
+
+// The four signed bytes of a word as floats (element e in bits 8e..8e+7,
+// other/int8-gemm.js:36-43).
+__device__ __forceinline__ float4 bytes_to_float4(int w) {
+  return make_float4((float)((w << 24) >> 24), (float)((w << 16) >> 24), (float)((w << 8) >> 24), (float)(w >> 24));
+}
 
 // Calls f(std::integral_constant<int, wave>) so that everything derived from the
 // wave index is a compile-time constant inside f (one copy of the code per wave).
@@ -223,23 +231,28 @@ __device__ __forceinline__ void for_wave(int wave, F f) {
 
 // Requests the slab share of this wave: items [wave*IPW, wave*IPW + IPW) of the
 // workgroup's `nitems`; item j is 64 consecutive float4 (column j / S, segment j % S).
-template <class P, class WS>
-__device__ __forceinline__ void load_items(WS& ws, const float4* __restrict__ slab, const float* __restrict__ bias,
-                                           int nitems, int wg, int wave, int lane) {
-  const float4* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
+__device__ __forceinline__ int ld_stream(const int* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void zero_item(float4& v) { v = make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ void zero_item(int& v) { v = 0; }
+
+template <class P, class WS, class T>
+__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, const float* __restrict__ bias,
+                                           const float* __restrict__ scale, int nitems, int wg, int wave, int lane) {
+  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
   for_wave(wave, [&](auto W) {
     constexpr int J0 = decltype(W)::value * P::IPW;
 #pragma unroll
     for (int i = 0; i < P::IPW; ++i) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      zero_item(ws.w[i]);
       if (J0 + i < P::ITEMS) {
-        if (!P::RAGGED || J0 + i < nitems) v = ld_stream(wgbase + (J0 + i) * 64);
+        if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
       }
-      ws.w[i] = v;
     }
   });
   const int t = opaque(threadIdx.x);
-  ws.bias = (t < P::CPW && wg * P::CPW + t < P::N) ? bias[wg * P::CPW + t] : 0.f;
+  const bool mine = t < P::CPW && wg * P::CPW + t < P::N;
+  ws.bias = mine ? bias[wg * P::CPW + t] : 0.f;
+  if (std::is_same<T, int>::value) ws.cscale = mine ? scale[wg * P::CPW + t] / 127.0f : 0.f;
 }
 
 // Requests the LayerNorm parameters of this lane's four elements of every segment.
@@ -255,61 +268,61 @@ __device__ __forceinline__ void load_ln(WS& ws, const float* __restrict__ gamma,
   }
 }
 
+__device__ __forceinline__ float4 to_float4(const float4& v) { return v; }
+__device__ __forceinline__ float4 to_float4(int v) { return bytes_to_float4(v); }
+
 // This wave's share of the matrix-vector product. The input row is read from xs
-// (LDS, zero padded up to S*SEG) into registers; with LNORM it is first normalised
-// there (instructions.js:451-550: biased variance about the mean, eps inside the
-// sqrt; the quotient (x - mean) / stdev is formed as (x - mean) * (1 / stdev)).
-// Every wave derives the two statistics itself, so no barrier is needed. Per
+// (LDS, zero padded up to S*SEG); with LNORM it is first normalised in registers
+// (instructions.js:451-550: biased variance about the mean, eps inside the sqrt;
+// the quotient (x - mean) / stdev is formed as (x - mean) * (1 / stdev)). Every wave
+// derives the two statistics itself, so the LayerNorm needs no barrier. Per
 // (column, wave) partial sums go to part[col*NW + wave].
+// The item code exists once per wave with every index a constant: a phase is short,
+// and what it costs is instruction count (a runtime-indexed single copy measured
+// 5-15 % slower at d = 1280 and 1600).
 template <class P, bool LNORM, class WS>
-__device__ __forceinline__ void gemv_items(const WS& ws, const float* xs, float* part, int nitems, int wave, int lane) {
+__device__ __forceinline__ void gemv_items(const WS& ws, float* xs, float* part, int nitems, int wave, int lane) {
   constexpr int S = P::S;
-  const float* xl = xs + opaque(lane) * 4;
+  float* xl = xs + opaque(lane) * 4;
+  constexpr int SR = LNORM ? S : 1;
+  float4 xr[SR];
+  if (LNORM) {
+    float sum = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < S; ++s2) {
+      xr[s2] = *reinterpret_cast<const float4*>(xl + s2 * SEG);
+      sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
+    }
+    const float mean = wave_sum(sum) / (float)P::K;
+    float q = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < S; ++s2) {
+      // lanes beyond K hold zeros that must not count as (0 - mean)^2
+      const bool in = s2 * SEG + SEG <= P::K || s2 * SEG + lane * 4 < P::K;
+      xr[s2].x -= mean; xr[s2].y -= mean; xr[s2].z -= mean; xr[s2].w -= mean;
+      const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
+      q += in ? qq : 0.f;
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)P::K + 1e-5f);
+#pragma unroll
+    for (int s2 = 0; s2 < S; ++s2) {
+      xr[s2].x = ws.g[s2].x * (xr[s2].x * rstd) + ws.b[s2].x;
+      xr[s2].y = ws.g[s2].y * (xr[s2].y * rstd) + ws.b[s2].y;
+      xr[s2].z = ws.g[s2].z * (xr[s2].z * rstd) + ws.b[s2].z;
+      xr[s2].w = ws.g[s2].w * (xr[s2].w * rstd) + ws.b[s2].w;
+    }
+  }
   for_wave(wave, [&](auto W) {
     constexpr int WV = decltype(W)::value;
     constexpr int J0 = WV * P::IPW;
-    // segments this wave needs: all of them for the statistics, else those of its items
-    float4 xr[S];
-#pragma unroll
-    for (int s2 = 0; s2 < S; ++s2) {
-      bool used = LNORM;
-      for (int i = 0; i < P::IPW; ++i)
-        if (J0 + i < P::ITEMS && (J0 + i) % S == s2) used = true;
-      xr[s2] = used ? *reinterpret_cast<const float4*>(xl + s2 * SEG) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    if (LNORM) {
-      float sum = 0.f;
-#pragma unroll
-      for (int s2 = 0; s2 < S; ++s2) sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
-      const float mean = wave_sum(sum) / (float)P::K;
-      float q = 0.f;
-#pragma unroll
-      for (int s2 = 0; s2 < S; ++s2) {
-        // lanes beyond K hold zeros that must not count as (0 - mean)^2
-        const bool in = s2 * SEG + SEG <= P::K || s2 * SEG + lane * 4 < P::K;
-        xr[s2].x -= mean; xr[s2].y -= mean; xr[s2].z -= mean; xr[s2].w -= mean;
-        const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
-        q += in ? qq : 0.f;
-      }
-      const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)P::K + 1e-5f);
-#pragma unroll
-      for (int s2 = 0; s2 < S; ++s2) {
-        xr[s2].x = ws.g[s2].x * (xr[s2].x * rstd) + ws.b[s2].x;
-        xr[s2].y = ws.g[s2].y * (xr[s2].y * rstd) + ws.b[s2].y;
-        xr[s2].z = ws.g[s2].z * (xr[s2].z * rstd) + ws.b[s2].z;
-        xr[s2].w = ws.g[s2].w * (xr[s2].w * rstd) + ws.b[s2].w;
-      }
-    }
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < P::IPW; ++i) {
-      constexpr int dummy = 0;
-      (void)dummy;
       if (J0 + i < P::ITEMS) {
         if (!P::RAGGED || J0 + i < nitems) {
           const int seg = (J0 + i) % S, col = (J0 + i) / S;
-          const float4 x = xr[seg];
-          const float4 w = ws.w[i];
+          const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
+          const float4 w = to_float4(ws.w[i]);
           acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
           if (seg == S - 1 || i == P::IPW - 1 || J0 + i == P::ITEMS - 1) {
             const float r = wave_sum(acc);
@@ -331,6 +344,13 @@ __device__ __forceinline__ float column_sum(const float* part, int c) {
   float s = 0.f;
   for (int v = v0; v <= v1; ++v) s += part[c * NW + v];
   return s;
+}
+
+// Finished value of local column c: partial sums, the int8 column scale, the bias last.
+template <class P, bool I8, class WS>
+__device__ __forceinline__ float colval(const float* part, int c, const WS& ws) {
+  const float s = column_sum<P>(part, c);
+  return (I8 ? s * ws.cscale : s) + ws.bias;
 }
 
 #ifdef WGPT_TRACE
@@ -402,12 +422,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   const int ah = wg / SPLIT, as = wg - ah * SPLIT;
 
   const LayerParamOffsets po = layer_param_offsets(D);
-  WSet<MAXI, C::SD> ws;
+  WSet<MAXI, C::SD, C::I8> ws;
+  typedef typename std::conditional<C::I8, int, float4>::type Item;
+  const Item* slabs = reinterpret_cast<const Item*>(a.slabs);
   float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
   int tok = a.tok[0];
 
-  load_items<PA>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+  load_items<PA>(ws, slabs, a.lparams + po.bA, a.lparams + po.sA, nitA, wg, wave, lane);
   load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
 
   for (int step = 0; step < a.nsteps; ++step) {
@@ -429,7 +451,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     float own_r = 0.f;  // residual stream value of the column this thread finishes in the d-wide phases
 
     for (int li = 0; li < a.L; ++li) {
-      const float4* slab = a.slabs + (size_t)li * a.slab_stride;
+      const Item* slab = slabs + (size_t)li * a.slab_stride;
       const float* lp = a.lparams + (size_t)li * po.stride;
       float* Kc = a.kv + ((size_t)(li * 2 + 0) * H + ah) * a.ctx * HS;
       float* Vc = a.kv + ((size_t)(li * 2 + 1) * H + ah) * a.ctx * HS;
@@ -450,9 +472,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         ++ep;
         if (tid < PA::CPW && wg * PA::CPW + tid < PA::N)
-          publish(a.bufQKV + wg * PA::CPW + tid, column_sum<PA>(part, tid) + ws.bias, ep);
+          publish(a.bufQKV + wg * PA::CPW + tid, colval<PA, C::I8>(part, tid, ws), ep);
         TRACE5(4);
-        load_items<PC>(ws, slab + a.slab_offC, lp + po.bC, nitC, wg, wave, lane);
+        load_items<PC>(ws, slab + a.slab_offC, lp + po.bC, lp + po.sC, nitC, wg, wave, lane);
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -605,11 +627,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         ++ep;
         if (tid < PC::CPW && wg * PC::CPW + tid < D) {
-          own_r += column_sum<PC>(part, tid) + ws.bias;  // model.js:159
+          own_r += colval<PC, C::I8>(part, tid, ws);  // model.js:159
           publish(a.bufR1 + wg * PC::CPW + tid, own_r, ep);
         }
         TRACE5(4);
-        load_items<PD>(ws, slab + a.slab_offD, lp + po.bD, nitD, wg, wave, lane);
+        load_items<PD>(ws, slab + a.slab_offD, lp + po.bD, lp + po.sD, nitD, wg, wave, lane);
         load_ln<D>(ws, lp + po.ln2g, lp + po.ln2b, lane);
         TRACE5(5);
       }
@@ -627,9 +649,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         ++ep;
         if (tid < PD::CPW && wg * PD::CPW + tid < HID)
-          publish(a.bufH + wg * PD::CPW + tid, gelu_ref(column_sum<PD>(part, tid) + ws.bias), ep);  // model.js:188
+          publish(a.bufH + wg * PD::CPW + tid, gelu_ref(colval<PD, C::I8>(part, tid, ws)), ep);  // model.js:188
         TRACE5(4);
-        load_items<PE>(ws, slab + a.slab_offE, lp + po.bE, nitE, wg, wave, lane);
+        load_items<PE>(ws, slab + a.slab_offE, lp + po.bE, lp + po.sE, nitE, wg, wave, lane);
         TRACE5(5);
       }
 
@@ -646,11 +668,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         ++ep;
         if (tid < PC::CPW && wg * PC::CPW + tid < D)
-          publish(a.bufR2 + wg * PC::CPW + tid, own_r + column_sum<PE>(part, tid) + ws.bias, ep);  // model.js:205
+          publish(a.bufR2 + wg * PC::CPW + tid, own_r + colval<PE, C::I8>(part, tid, ws), ep);  // model.js:205
         TRACE5(4);
         // next layer's c_attn share, or the first layer's for the next step
         if (li + 1 < a.L) {
-          load_items<PA>(ws, slab + a.slab_stride, lp + po.stride + po.bA, nitA, wg, wave, lane);
+          load_items<PA>(ws, slab + a.slab_stride, lp + po.stride + po.bA, lp + po.stride + po.sA, nitA, wg, wave, lane);
           load_ln<D>(ws, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b, lane);
         } else {
           load_ln<D>(ws, a.lnf_g, a.lnf_b, lane);
@@ -752,7 +774,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
     TRACE(2 + a.L * 8);
     if (step + 1 < a.nsteps) {
-      load_items<PA>(ws, a.slabs, a.lparams + po.bA, nitA, wg, wave, lane);
+      load_items<PA>(ws, slabs, a.lparams + po.bA, a.lparams + po.sA, nitA, wg, wave, lane);
       load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
@@ -804,6 +826,29 @@ __global__ void build_slab_kernel(const float* __restrict__ W, int ldw, int K, i
   slab[idx] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+// int8: item (w, j = c*S + seg, lane) is one word holding rows k..k+3 (k = seg*256 + lane*4)
+// of column w*cpw + c, gathered from the reference packing [K, N/4] (4 consecutive
+// columns per word, other/int8-gemm.js:36-43).
+__global__ void build_slab_i8_kernel(const int32_t* __restrict__ Wq, int ldwq, int K, int N, int cpw, int S, size_t total,
+                                     int32_t* __restrict__ slab) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int lane = (int)(idx & 63);
+  const size_t it = idx >> 6;
+  const int per_wg = cpw * S;
+  const int w = (int)(it / per_wg), j = (int)(it - (size_t)w * per_wg);
+  const int c = j / S, seg = j - c * S;
+  const int col = w * cpw + c, k = seg * SEG + lane * 4;
+  unsigned out = 0;
+  if (col < N)
+    for (int e = 0; e < 4; ++e)
+      if (k + e < K) {
+        const unsigned word = (unsigned)Wq[(size_t)(k + e) * ldwq + (col >> 2)];
+        out |= ((word >> (8 * (col & 3))) & 0xffu) << (8 * e);
+      }
+  slab[idx] = (int32_t)out;
+}
+
 template <class C>
 size_t lds_bytes_of() {
   typedef Phases<C> PS;
@@ -850,14 +895,22 @@ hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4
   return hipGetLastError();
 }
 
-bool persistent_supports(int d, int n_head, int n_ctx) {
+hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g, int32_t* slab, hipStream_t s) {
+  const size_t total = slab_float4s(g);
+  build_slab_i8_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(Wq, ldwq, K, g.N, g.cpw, g.S, total, slab);
+  return hipGetLastError();
+}
+
+bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
   if (((n_ctx + PD_SPLIT - 1) / PD_SPLIT + 31) / 32 > PD_MAXKV) return false;
+  if (weight_dtype == 1) return d == 1600 && n_head == 25;
   return (d == 384 && n_head == 6) || (d == 768 && n_head == 12) || (d == 1024 && n_head == 16) ||
          (d == 1280 && n_head == 20);
 }
 
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
-  if (!persistent_supports(a.d, a.H, a.ctx)) return hipErrorInvalidValue;
+  if (!persistent_supports(a.d, a.H, a.ctx, a.weight_dtype)) return hipErrorInvalidValue;
+  if (a.weight_dtype == 1) return launch_t<Shape<1600, 25, true>>(a, s);
   switch (a.d) {
     case 384: return launch_t<Shape<384, 6>>(a, s);
     case 768: return launch_t<Shape<768, 12>>(a, s);

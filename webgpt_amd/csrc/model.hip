@@ -186,12 +186,14 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 static int setup_persistent(Model* m) {
   m->persist_ok = false;
   const int d = m->d, hid = 4 * d, G = PD_GRID, split = PD_SPLIT;
-  if (m->p.weight_dtype != 0 || m->hs != 64) return WGPT_OK;
+  const bool i8 = m->p.weight_dtype == 1;
+  if (m->hs != 64) return WGPT_OK;
   if (rt().compute_units < G) return WGPT_OK;
-  if (!persistent_supports(d, m->H, m->ctx)) return WGPT_OK;
+  if (!persistent_supports(d, m->H, m->ctx, m->p.weight_dtype)) return WGPT_OK;
   PersistentArgs& a = m->pa;
   a = PersistentArgs{};
   a.L = m->L; a.H = m->H; a.d = d; a.ctx = m->ctx; a.V = m->V;
+  a.weight_dtype = m->p.weight_dtype;
   a.scale = (float)(1.0 / std::sqrt((double)m->hs));
   const PhaseGeom gA = make_geom(3 * d, d), gC = make_geom(d, d), gD = make_geom(hid, d), gE = make_geom(d, hid);
   a.rows_per_wg = (m->V + G - 1) / G;
@@ -203,24 +205,36 @@ static int setup_persistent(Model* m) {
   a.slab_offD = a.slab_offC + slab_float4s(gC);
   a.slab_offE = a.slab_offD + slab_float4s(gD);
   a.slab_stride = a.slab_offE + slab_float4s(gE);
-  float4* slabs;
-  if ((rc = dev_alloc(m, a.slab_stride * (size_t)m->L * sizeof(float4), (void**)&slabs))) return rc;
+  // an item lane is a float4 (fp32) or one word of four int8 (int8)
+  const size_t lane_bytes = i8 ? sizeof(int32_t) : sizeof(float4);
+  char* slabs;
+  if ((rc = dev_alloc(m, a.slab_stride * (size_t)m->L * lane_bytes, (void**)&slabs))) return rc;
   const LayerParamOffsets po = layer_param_offsets(d);
   float* lparams;
   if ((rc = dev_alloc(m, sizeof(float) * (size_t)po.stride * m->L, (void**)&lparams))) return rc;
   for (int i = 0; i < m->L; ++i) {
     const LayerW& l = m->layers[i];
-    float4* sl = slabs + (size_t)i * a.slab_stride;
-    LAUNCH(build_slab(l.attn.w, 3 * d, d, gA, sl, rt().stream));
-    LAUNCH(build_slab(l.proj.w, d, d, gC, sl + a.slab_offC, rt().stream));
-    LAUNCH(build_slab(l.fc.w, hid, d, gD, sl + a.slab_offD, rt().stream));
-    LAUNCH(build_slab(l.fc2.w, d, hid, gE, sl + a.slab_offE, rt().stream));
+    char* slb = slabs + (size_t)i * a.slab_stride * lane_bytes;
+    if (i8) {
+      int32_t* sl = (int32_t*)slb;
+      LAUNCH(build_slab_i8(l.attn.q, 3 * d / 4, d, gA, sl, rt().stream));
+      LAUNCH(build_slab_i8(l.proj.q, d / 4, d, gC, sl + a.slab_offC, rt().stream));
+      LAUNCH(build_slab_i8(l.fc.q, hid / 4, d, gD, sl + a.slab_offD, rt().stream));
+      LAUNCH(build_slab_i8(l.fc2.q, d / 4, hid, gE, sl + a.slab_offE, rt().stream));
+    } else {
+      float4* sl = (float4*)slb;
+      LAUNCH(build_slab(l.attn.w, 3 * d, d, gA, sl, rt().stream));
+      LAUNCH(build_slab(l.proj.w, d, d, gC, sl + a.slab_offC, rt().stream));
+      LAUNCH(build_slab(l.fc.w, hid, d, gD, sl + a.slab_offD, rt().stream));
+      LAUNCH(build_slab(l.fc2.w, d, hid, gE, sl + a.slab_offE, rt().stream));
+    }
     float* lp = lparams + (size_t)i * po.stride;
-    const struct { int off; const float* src; int n; } parts[8] = {
+    const struct { int off; const float* src; int n; } parts[12] = {
         {po.bA, l.attn_b, 3 * d}, {po.bC, l.proj_b, d}, {po.bD, l.fc_b, hid}, {po.bE, l.fc2_b, d},
-        {po.ln1g, l.ln1_g, d},    {po.ln1b, l.ln1_b, d}, {po.ln2g, l.ln2_g, d}, {po.ln2b, l.ln2_b, d}};
+        {po.ln1g, l.ln1_g, d},    {po.ln1b, l.ln1_b, d}, {po.ln2g, l.ln2_g, d}, {po.ln2b, l.ln2_b, d},
+        {po.sA, l.attn.s, 3 * d}, {po.sC, l.proj.s, d}, {po.sD, l.fc.s, hid}, {po.sE, l.fc2.s, d}};
     for (const auto& pt : parts)
-      WGPT_HIP(hipMemcpyAsync(lp + pt.off, pt.src, sizeof(float) * pt.n, hipMemcpyDeviceToDevice, rt().stream));
+      if (pt.src) WGPT_HIP(hipMemcpyAsync(lp + pt.off, pt.src, sizeof(float) * pt.n, hipMemcpyDeviceToDevice, rt().stream));
   }
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   a.slabs = slabs;
@@ -574,7 +588,7 @@ int wgpt_model_set_decode_mode(wgpt_model h, int mode) {
   if (mode != 0 && mode != 1) return fail(WGPT_ERR_ARG, "wgpt_model_set_decode_mode: unknown mode %d", mode);
   if (mode == 1 && !m->persist_ok)
     return fail(WGPT_ERR_STATE, "wgpt_model_set_decode_mode: the persistent decode path is not available for this model "
-                                "(needs fp32 weights, head size 64, 256 compute units)");
+                                "(needs head size 64, a supported width and 256 compute units)");
   m->decode_mode = mode;
   return WGPT_OK;
 }
