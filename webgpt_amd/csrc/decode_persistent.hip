@@ -111,9 +111,18 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// Hardware approximations (about 1 ulp each), used where an exact quotient, square
+// root or exponential would put a dozen dependent instructions on a phase's
+// critical path; the difference is orders of magnitude inside the parity tolerance.
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 __device__ __forceinline__ float gelu_ref(float x) {  // instructions.js:718-727
   const float x3 = x * x * x;
-  const float cdf = 0.5f * (1.0f + tanhf(0.7978845608f * (x + 0.044715f * x3)));
+  // 1 + tanh(u) = 2 - 2 / (1 + exp(2u)); exp overflowing to +inf gives exactly 2, underflowing to 0 gives 0
+  const float u = 0.7978845608f * (x + 0.044715f * x3);
+  const float cdf = 1.0f - fast_rcp(1.0f + fast_exp(2.0f * u));
   float r = x * cdf;
   r = x < -10.0f ? 0.0f : r;
   r = x > 10.0f ? x : r;
@@ -164,6 +173,9 @@ struct Phase {
 // Polls N {value, epoch} words until all carry `epoch`, storing the values to dst
 // (LDS). All loads of a round are issued before any is tested. On SPIN_LIMIT rounds,
 // or when another thread or workgroup has already given up, raises sh.bail.
+#ifndef WGPT_POLL_DELAY
+#define WGPT_POLL_DELAY 0
+#endif
 template <int N>
 __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err) {
   constexpr int NP = (N + NT - 1) / NT;
@@ -173,6 +185,9 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
   for (int i = 0; i < NP; ++i)
     if (i * NT + NT <= N || t + i * NT < N) pending |= 1u << i;
   unsigned spins = 0;
+#if WGPT_POLL_DELAY > 0
+  __builtin_amdgcn_s_sleep(WGPT_POLL_DELAY);
+#endif
   while (pending) {
     u64 pk[NP];
 #pragma unroll
@@ -245,7 +260,7 @@ __device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, c
     for (int i = 0; i < P::IPW; ++i) {
       zero_item(ws.w[i]);
       if (J0 + i < P::ITEMS) {
-        if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
+        if ((!P::RAGGED || J0 + i < nitems) && !(WGPT_DBG_SKIP_W && nitems >= 0)) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
       }
     }
   });
@@ -293,7 +308,7 @@ __device__ __forceinline__ void gemv_items(const WS& ws, float* xs, float* part,
       xr[s2] = *reinterpret_cast<const float4*>(xl + s2 * SEG);
       sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
     }
-    const float mean = wave_sum(sum) / (float)P::K;
+    const float mean = wave_sum(sum) * (1.0f / (float)P::K);
     float q = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
@@ -303,7 +318,7 @@ __device__ __forceinline__ void gemv_items(const WS& ws, float* xs, float* part,
       const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
       q += in ? qq : 0.f;
     }
-    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)P::K + 1e-5f);
+    const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)P::K) + 1e-5f);
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
       xr[s2].x = ws.g[s2].x * (xr[s2].x * rstd) + ws.b[s2].x;
@@ -399,7 +414,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float* attp = xs + XS;      // [ATTP]
   float* part = attp + ATTP;  // [PART]
   float* qkv_s = part + PART; // [3*HS]
-  float* hw = qkv_s + 3 * HS; // [H*SPLIT] per-slice merge weights
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
@@ -520,7 +534,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
         }
         __syncthreads();
-        if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + 5);
         // the slice that holds the new position appends it to the cache and uses it from LDS
@@ -559,7 +572,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 #pragma unroll
           for (int i = 0; i < MAXKV; ++i) {
             if (i < nkv) {
-              const float p = sc[i] > -INFINITY ? expf(sc[i] - m) : 0.f;
+              const float p = sc[i] > -INFINITY ? fast_exp(sc[i] - m) : 0.f;
               l += p;
               o.x += p * vreg[i].x; o.y += p * vreg[i].y; o.z += p * vreg[i].z; o.w += p * vreg[i].w;
             }
@@ -587,37 +600,32 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         constexpr int PH = PH_PROJ;
         poll_words<C::ATTW>(a.bufATT, ep, attp, a.err);
         __syncthreads();
-        if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        // per (head, slice): weight exp(m_s - M) / L of the slice's unnormalised output
-        if (tid < H) {
-          const float* phd = attp + tid * SPLIT * (HS + 2);
-          float M = -INFINITY;
-#pragma unroll
-          for (int s2 = 0; s2 < SPLIT; ++s2) M = fmaxf(M, phd[s2 * (HS + 2) + HS]);
-          float wv[SPLIT];
-          float Lsum = 0.f;
-#pragma unroll
-          for (int s2 = 0; s2 < SPLIT; ++s2) {
-            const float ms = phd[s2 * (HS + 2) + HS];
-            wv[s2] = ms > -INFINITY ? expf(ms - M) : 0.f;
-            Lsum += phd[s2 * (HS + 2) + HS + 1] * wv[s2];
-          }
-#pragma unroll
-          for (int s2 = 0; s2 < SPLIT; ++s2) hw[tid * SPLIT + s2] = wv[s2] / Lsum;
-        }
-        __syncthreads();
+        // merge of the slices of each head (flash-decoding): element e of head h is
+        // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
+        // derives the weights of its head itself (broadcast LDS reads, no barrier)
 #pragma unroll
         for (int k = 0; k < (D + NT - 1) / NT; ++k) {
           const int e = tid + k * NT;
           if (k * NT + NT <= D || e < D) {
             const int h = e / HS, c = e - h * HS;
-            const float* phd = attp + h * SPLIT * (HS + 2) + c;
-            float val = 0.f;
+            const float* phd = attp + h * SPLIT * (HS + 2);
+            float ms[SPLIT];
+            float M = -INFINITY;
 #pragma unroll
-            for (int s2 = 0; s2 < SPLIT; ++s2) val += phd[s2 * (HS + 2)] * hw[h * SPLIT + s2];
-            xs[e] = val;
+            for (int s2 = 0; s2 < SPLIT; ++s2) {
+              ms[s2] = phd[s2 * (HS + 2) + HS];
+              M = fmaxf(M, ms[s2]);
+            }
+            float Lsum = 0.f, val = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < SPLIT; ++s2) {
+              const float wv = ms[s2] > -INFINITY ? fast_exp(ms[s2] - M) : 0.f;
+              Lsum += phd[s2 * (HS + 2) + HS + 1] * wv;
+              val += phd[s2 * (HS + 2) + c] * wv;
+            }
+            xs[e] = val * fast_rcp(Lsum);
           }
         }
         __syncthreads();
@@ -641,7 +649,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         constexpr int PH = PH_FC;
         poll_words<D>(a.bufR1, ep, xs, a.err);
         __syncthreads();
-        if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + PH);
         gemv_items<PD, true>(ws, xs, part, nitD, wave, lane);
@@ -660,7 +667,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         constexpr int PH = PH_FC2;
         poll_words<HID>(a.bufH, ep, xs, a.err);
         __syncthreads();
-        if (sh.bail) return;
         wait_loads();
         TRACE(1 + li * 8 + PH);
         gemv_items<PE, false>(ws, xs, part, nitE, wave, lane);
@@ -705,7 +711,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           xv[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
           sum += (xv[s2].x + xv[s2].y) + (xv[s2].z + xv[s2].w);
         }
-        const float mean = wave_sum(sum) / (float)D;
+        const float mean = wave_sum(sum) * (1.0f / (float)D);
         float q = 0.f;
 #pragma unroll
         for (int s2 = 0; s2 < S; ++s2) {
@@ -714,7 +720,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           const float qq = (xv[s2].x * xv[s2].x + xv[s2].y * xv[s2].y) + (xv[s2].z * xv[s2].z + xv[s2].w * xv[s2].w);
           q += in ? qq : 0.f;
         }
-        const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)D + 1e-5f);
+        const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)D) + 1e-5f);
 #pragma unroll
         for (int s2 = 0; s2 < S; ++s2) {
           xv[s2].x = ws.g[s2].x * (xv[s2].x * rstd) + ws.b[s2].x;
