@@ -63,8 +63,11 @@ struct PersistentArgs {
 
 PhaseGeom make_geom(int N, int K);
 size_t slab_float4s(const PhaseGeom& g);
-// Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g.
-hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4* slab, hipStream_t s);
+// Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g; with rowscale
+// (the gamma of the LayerNorm in front of the matrix, or null) as diag(rowscale) W.
+hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const float* rowscale, float4* slab, hipStream_t s);
+// out[N] = bias + beta W: the beta of that LayerNorm folded into the bias.
+hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* beta, const float* bias, float* out, hipStream_t s);
 // Same for int8 words Wq[K, ldwq] (4 columns per word): one word per item lane.
 hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g, int32_t* slab, hipStream_t s);
 // Model shapes the persistent kernel is instantiated for.

@@ -160,19 +160,25 @@ struct Shape {
 };
 
 // One linear phase: N outputs from a K-long input.
-template <int N_, int K_>
+// WHOLE: local column c of a workgroup lives in wave c % NW (as its (c / NW)-th),
+// which holds all S items of the column and finishes it (scale, bias, activation) in
+// lane c / NW; the finished values meet in LDS so that one wave publishes them with
+// one store instruction (a store per wave makes the hop measurably slower).
+// Otherwise (the long contraction of the second MLP matrix) the workgroup's items
+// are dealt to the waves in runs of IPW, a column is the sum of the partials of
+// several waves and thread c finishes column c.
+template <int N_, int K_, bool WHOLE_>
 struct Phase {
   static constexpr int N = N_, K = K_;
+  static constexpr bool WHOLE = WHOLE_;
   static constexpr int CPW = (N + PD_GRID - 1) / PD_GRID;  // columns per workgroup
-  static constexpr int S = (K + SEG - 1) / SEG;            // segments per column
+  static constexpr int S = (K + SEG - 1) / SEG;            // segments (items) per column
   static constexpr int ITEMS = CPW * S;                    // items per workgroup
-  static constexpr int IPW = (ITEMS + NW - 1) / NW;        // items per wave
+  static constexpr int CW = (CPW + NW - 1) / NW;           // columns finished per wave
+  static constexpr int IPW = WHOLE ? CW * S : (ITEMS + NW - 1) / NW;  // items per wave
   static constexpr bool RAGGED = CPW * PD_GRID != N;       // some workgroups finish fewer than CPW columns
 };
 
-// Polls N {value, epoch} words until all carry `epoch`, storing the values to dst
-// (LDS). All loads of a round are issued before any is tested. On SPIN_LIMIT rounds,
-// or when another thread or workgroup has already given up, raises sh.bail.
 #ifndef WGPT_POLL_DELAY
 #define WGPT_POLL_DELAY 0
 #endif
@@ -211,15 +217,13 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
   }
 }
 
-// Registers of one linear phase: this wave's share of the weight slab (MAXI float4
-// per lane), the bias of the column this thread finishes, and the LayerNorm
-// parameters of the lane's elements of every segment (phases with a LayerNorm).
-template <int MAXI, int SD, bool I8>
+// Registers of one linear phase: this wave's share of the weight slab (MAXI items per
+// lane) and the bias (int8: also scale / 127) of the column this lane finishes.
+template <int MAXI, bool I8>
 struct WSet {
   typename std::conditional<I8, int, float4>::type w[MAXI];  // an int8 item is one word per lane
   float bias;
-  float cscale;  // int8: scale[column] / 127 of the column this thread finishes
-  float4 g[SD], b[SD];
+  float cscale;
 };
 
 // The four signed bytes of a word as floats (element e in bits 8e..8e+7,
@@ -244,89 +248,155 @@ __device__ __forceinline__ void for_wave(int wave, F f) {
   }
 }
 
-// Requests the slab share of this wave: items [wave*IPW, wave*IPW + IPW) of the
-// workgroup's `nitems`; item j is 64 consecutive float4 (column j / S, segment j % S).
 __device__ __forceinline__ int ld_stream(const int* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void zero_item(float4& v) { v = make_float4(0.f, 0.f, 0.f, 0.f); }
 __device__ __forceinline__ void zero_item(int& v) { v = 0; }
-
-template <class P, class WS, class T>
-__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, const float* __restrict__ bias,
-                                           const float* __restrict__ scale, int nitems, int wg, int wave, int lane) {
-  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
-  for_wave(wave, [&](auto W) {
-    constexpr int J0 = decltype(W)::value * P::IPW;
-#pragma unroll
-    for (int i = 0; i < P::IPW; ++i) {
-      zero_item(ws.w[i]);
-      if (J0 + i < P::ITEMS) {
-        if ((!P::RAGGED || J0 + i < nitems) && !(WGPT_DBG_SKIP_W && nitems >= 0)) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
-      }
-    }
-  });
-  const int t = opaque(threadIdx.x);
-  const bool mine = t < P::CPW && wg * P::CPW + t < P::N;
-  ws.bias = mine ? bias[wg * P::CPW + t] : 0.f;
-  if (std::is_same<T, int>::value) ws.cscale = mine ? scale[wg * P::CPW + t] / 127.0f : 0.f;
-}
-
-// Requests the LayerNorm parameters of this lane's four elements of every segment.
-template <int D, class WS>
-__device__ __forceinline__ void load_ln(WS& ws, const float* __restrict__ gamma, const float* __restrict__ beta, int lane) {
-  constexpr int S = (D + SEG - 1) / SEG;
-  const int k0 = opaque(lane) * 4;
-#pragma unroll
-  for (int s2 = 0; s2 < S; ++s2) {
-    const bool in = s2 * SEG + SEG <= D || s2 * SEG + k0 < D;
-    ws.g[s2] = in ? *reinterpret_cast<const float4*>(gamma + s2 * SEG + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
-    ws.b[s2] = in ? *reinterpret_cast<const float4*>(beta + s2 * SEG + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
-  }
-}
-
 __device__ __forceinline__ float4 to_float4(const float4& v) { return v; }
 __device__ __forceinline__ float4 to_float4(int v) { return bytes_to_float4(v); }
 
-// This wave's share of the matrix-vector product. The input row is read from xs
-// (LDS, zero padded up to S*SEG); with LNORM it is first normalised in registers
-// (instructions.js:451-550: biased variance about the mean, eps inside the sqrt;
-// the quotient (x - mean) / stdev is formed as (x - mean) * (1 / stdev)). Every wave
-// derives the two statistics itself, so the LayerNorm needs no barrier. Per
-// (column, wave) partial sums go to part[col*NW + wave].
-// The item code exists once per wave with every index a constant: a phase is short,
-// and what it costs is instruction count (a runtime-indexed single copy measured
-// 5-15 % slower at d = 1280 and 1600).
-template <class P, bool LNORM, class WS>
-__device__ __forceinline__ void gemv_items(const WS& ws, float* xs, float* part, int nitems, int wave, int lane) {
-  constexpr int S = P::S;
-  float* xl = xs + opaque(lane) * 4;
-  constexpr int SR = LNORM ? S : 1;
-  float4 xr[SR];
+// Requests this wave's items of the workgroup's slab share into registers; item
+// j = c * S + seg of the workgroup is 64 consecutive lanes' worth (a float4, or one
+// word of four int8, per lane) of segment seg of local column c. `ncols` is the
+// number of columns this workgroup finishes (CPW except at the ragged end).
+template <class P, class WS, class T>
+__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, const float* __restrict__ bias,
+                                           const float* __restrict__ scale, int ncols, int wg, int wave, int lane) {
+  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
+  if (P::WHOLE) {
+#pragma unroll
+    for (int cc = 0; cc < P::CW; ++cc) {
+      const int c = wave + cc * NW;
+#pragma unroll
+      for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
+      if (c < (P::RAGGED ? ncols : P::CPW)) {
+#pragma unroll
+        for (int seg = 0; seg < P::S; ++seg) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);
+      }
+    }
+  } else {
+    const int nitems = ncols * P::S;
+    for_wave(wave, [&](auto W) {
+      constexpr int J0 = decltype(W)::value * P::IPW;
+#pragma unroll
+      for (int i = 0; i < P::IPW; ++i) {
+        zero_item(ws.w[i]);
+        if (J0 + i < P::ITEMS) {
+          if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
+        }
+      }
+    });
+  }
+  // the lane that finishes a column: lane cc of the wave that holds it (WHOLE), else thread c
+  const int l = opaque(lane);
+  const int c = P::WHOLE ? wave + l * NW : (int)threadIdx.x;
+  const bool mine = (P::WHOLE ? l < P::CW : true) && c < ncols;
+  ws.bias = mine ? bias[wg * P::CPW + c] : 0.f;
+  if (std::is_same<T, int>::value) ws.cscale = mine ? scale[wg * P::CPW + c] / 127.0f : 0.f;
+}
+
+// LayerNorm parameters travel global memory -> registers (requested with the weights
+// of the phase) -> LDS (deposited next to the polled input row, before the barrier
+// that follows the poll): gamma at lnp[0, D), beta at lnp[D, 2D).
+template <int D, int NLN>
+__device__ __forceinline__ void request_ln(float4 (&r)[NLN], const float* __restrict__ gamma, const float* __restrict__ beta) {
+  const int t = opaque(threadIdx.x);
+#pragma unroll
+  for (int i = 0; i < NLN; ++i) {
+    const int idx = t + i * NT;
+    r[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (idx < D / 4) r[i] = reinterpret_cast<const float4*>(gamma)[idx];
+    else if (idx < D / 2) r[i] = reinterpret_cast<const float4*>(beta)[idx - D / 4];
+  }
+}
+template <int D, int NLN>
+__device__ __forceinline__ void deposit_ln(const float4 (&r)[NLN], float* lnp) {
+  const int t = opaque(threadIdx.x);
+#pragma unroll
+  for (int i = 0; i < NLN; ++i)
+    if (t + i * NT < D / 2) reinterpret_cast<float4*>(lnp)[t + i * NT] = r[i];
+}
+
+// The input row (LDS, zero padded up to S * SEG) as this lane's float4 of every
+// segment; with LNORM normalised first (instructions.js:451-550: biased variance
+// about the mean, eps inside the square root). Every wave derives the two
+// statistics itself, so the LayerNorm needs no barrier. AFFINE applies gamma and
+// beta from lnp; without it the caller's weights hold diag(gamma) W and its bias
+// holds bias + beta W (eight waves re-reading 2*K parameters from LDS every phase
+// cost about a microsecond per LayerNorm).
+template <int K, bool LNORM, bool AFFINE>
+__device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], const float* xs, const float* lnp, int lane) {
+  constexpr int S = (K + SEG - 1) / SEG;
+  const int l4 = opaque(lane) * 4;
+#pragma unroll
+  for (int s2 = 0; s2 < S; ++s2) xr[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + l4);
   if (LNORM) {
     float sum = 0.f;
 #pragma unroll
-    for (int s2 = 0; s2 < S; ++s2) {
-      xr[s2] = *reinterpret_cast<const float4*>(xl + s2 * SEG);
-      sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
-    }
-    const float mean = wave_sum(sum) * (1.0f / (float)P::K);
+    for (int s2 = 0; s2 < S; ++s2) sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
+    const float mean = wave_sum(sum) * (1.0f / (float)K);
     float q = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
       // lanes beyond K hold zeros that must not count as (0 - mean)^2
-      const bool in = s2 * SEG + SEG <= P::K || s2 * SEG + lane * 4 < P::K;
+      const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
       xr[s2].x -= mean; xr[s2].y -= mean; xr[s2].z -= mean; xr[s2].w -= mean;
       const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
       q += in ? qq : 0.f;
     }
-    const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)P::K) + 1e-5f);
+    const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)K) + 1e-5f);
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
-      xr[s2].x = ws.g[s2].x * (xr[s2].x * rstd) + ws.b[s2].x;
-      xr[s2].y = ws.g[s2].y * (xr[s2].y * rstd) + ws.b[s2].y;
-      xr[s2].z = ws.g[s2].z * (xr[s2].z * rstd) + ws.b[s2].z;
-      xr[s2].w = ws.g[s2].w * (xr[s2].w * rstd) + ws.b[s2].w;
+      const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
+      if (AFFINE) {
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 g = in ? *reinterpret_cast<const float4*>(lnp + s2 * SEG + l4) : z;
+        const float4 b = in ? *reinterpret_cast<const float4*>(lnp + K + s2 * SEG + l4) : z;
+        xr[s2].x = g.x * (xr[s2].x * rstd) + b.x;
+        xr[s2].y = g.y * (xr[s2].y * rstd) + b.y;
+        xr[s2].z = g.z * (xr[s2].z * rstd) + b.z;
+        xr[s2].w = g.w * (xr[s2].w * rstd) + b.w;
+      } else {
+        // gamma and beta live in the weights and the bias; padding lanes meet zero weights
+        xr[s2].x *= rstd; xr[s2].y *= rstd; xr[s2].z *= rstd; xr[s2].w *= rstd;
+      }
     }
   }
+}
+
+// WHOLE phases: the dot products of this wave's columns; lane cc returns the sum of
+// the wave's cc-th column (local column wave + cc * NW), before scale and bias.
+template <class P, bool LNORM, bool AFFINE, class WS>
+__device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const float* lnp, int ncols, int wave, int lane) {
+  static_assert(P::WHOLE, "phase is not laid out by whole columns");
+  float4 xr[P::S];
+  input_row<P::K, LNORM, AFFINE>(xr, xs, lnp, lane);
+  float val = 0.f;
+#pragma unroll
+  for (int cc = 0; cc < P::CW; ++cc) {
+    if (wave + cc * NW < (P::RAGGED ? ncols : P::CPW)) {
+      float acc = 0.f;
+#pragma unroll
+      for (int seg = 0; seg < P::S; ++seg) {
+        const float4 w = to_float4(ws.w[cc * P::S + seg]);
+        acc += (w.x * xr[seg].x + w.y * xr[seg].y) + (w.z * xr[seg].z + w.w * xr[seg].w);
+      }
+      const float r = wave_sum(acc);
+      val = lane == cc ? r : val;
+    }
+  }
+  return val;
+}
+
+// Other phases: per (column, wave) partial sums go to part[col * NW + wave]. The item
+// code exists once per wave with every index a constant: a phase is short, and what
+// it costs is instruction count (a runtime-indexed single copy measured 5-15 %
+// slower at d = 1280 and 1600).
+template <class P, class WS>
+__device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float* part, int ncols, int wave, int lane) {
+  static_assert(!P::WHOLE, "phase is laid out by whole columns");
+  constexpr int S = P::S;
+  const float* xl = xs + opaque(lane) * 4;
+  const int nitems = ncols * S;
   for_wave(wave, [&](auto W) {
     constexpr int WV = decltype(W)::value;
     constexpr int J0 = WV * P::IPW;
@@ -336,7 +406,7 @@ __device__ __forceinline__ void gemv_items(const WS& ws, float* xs, float* part,
       if (J0 + i < P::ITEMS) {
         if (!P::RAGGED || J0 + i < nitems) {
           const int seg = (J0 + i) % S, col = (J0 + i) / S;
-          const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
+          const float4 x = *reinterpret_cast<const float4*>(xl + seg * SEG);
           const float4 w = to_float4(ws.w[i]);
           acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
           if (seg == S - 1 || i == P::IPW - 1 || J0 + i == P::ITEMS - 1) {
@@ -361,11 +431,10 @@ __device__ __forceinline__ float column_sum(const float* part, int c) {
   return s;
 }
 
-// Finished value of local column c: partial sums, the int8 column scale, the bias last.
-template <class P, bool I8, class WS>
-__device__ __forceinline__ float colval(const float* part, int c, const WS& ws) {
-  const float s = column_sum<P>(part, c);
-  return (I8 ? s * ws.cscale : s) + ws.bias;
+// Finished value of a column from its dot product: the int8 column scale, the bias last.
+template <bool I8, class WS>
+__device__ __forceinline__ float finish(float dot, const WS& ws) {
+  return (I8 ? dot * ws.cscale : dot) + ws.bias;
 }
 
 #ifdef WGPT_TRACE
@@ -385,15 +454,22 @@ __device__ __forceinline__ float colval(const float* part, int c, const WS& ws) 
 // Linear phases of a layer, in execution order.
 enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
 
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
 template <class C>
 struct Phases {
-  typedef Phase<3 * C::D, C::D> A;   // c_attn
-  typedef Phase<C::D, C::D> Cc;      // attention c_proj
-  typedef Phase<C::HID, C::D> Dd;    // c_fc
-  typedef Phase<C::D, C::HID> E;     // mlp c_proj
-  static constexpr int MAXI = (A::IPW > Dd::IPW ? A::IPW : Dd::IPW) > (Cc::IPW > E::IPW ? Cc::IPW : E::IPW)
-                                  ? (A::IPW > Dd::IPW ? A::IPW : Dd::IPW)
-                                  : (Cc::IPW > E::IPW ? Cc::IPW : E::IPW);
+  typedef Phase<3 * C::D, C::D, true> A;    // c_attn
+  typedef Phase<C::D, C::D, true> Cc;       // attention c_proj
+  typedef Phase<C::HID, C::D, true> Dd;     // c_fc
+  typedef Phase<C::D, C::HID, false> E;     // mlp c_proj
+  static constexpr int MAXI = cmax(cmax(A::IPW, Dd::IPW), cmax(Cc::IPW, E::IPW));
+  // Two register sets (c_attn and c_fc in one, the two projections in the other) let a
+  // phase's weights be requested a whole phase ahead, right after the poll of the
+  // phase before it; affordable while a set is at most 32 registers.
+#ifndef WGPT_DUAL_LIMIT
+#define WGPT_DUAL_LIMIT 32
+#endif
+  static constexpr bool DUAL = MAXI * (C::I8 ? 1 : 4) <= WGPT_DUAL_LIMIT;
 };
 
 template <class C, int MAXKV>
@@ -404,31 +480,43 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   typedef typename PS::Dd PD;
   typedef typename PS::E PE;
   constexpr int D = C::D, HS = C::HS, H = C::H, HID = C::HID, SPLIT = C::SPLIT, MAXI = PS::MAXI;
-  constexpr int XS = C::SH * SEG;                                   // floats of the input row buffer
+  constexpr bool DUAL = PS::DUAL, I8 = C::I8;
+  constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
+  constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
+  constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
   constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;     // floats of the staged exchange words
-  constexpr int CPWMAX = PA::CPW > PD::CPW ? PA::CPW : PD::CPW;
-  constexpr int PART = 32 * (HS + 4) > CPWMAX * NW ? 32 * (HS + 4) : CPWMAX * NW;
+  constexpr int PART = 32 * (HS + 4) > PE::CPW * NW ? 32 * (HS + 4) : PE::CPW * NW;
+  constexpr int NLN = (D / 2 + NT - 1) / NT;                        // float4 of LayerNorm parameters per thread
 
+  // Input rows alternate between two buffers (xs0: residual stream rows; xs1: merged
+  // attention output, MLP hidden row), so that a poll never writes the buffer the
+  // dot products of the phase before it may still be reading.
   extern __shared__ float lds[];
-  float* xs = lds;            // [XS]
-  float* attp = xs + XS;      // [ATTP]
-  float* part = attp + ATTP;  // [PART]
-  float* qkv_s = part + PART; // [3*HS]
+  float* xs0 = lds;            // [XS0]
+  float* xs1 = xs0 + XS0;      // [XS1]
+  float* lnp = xs1 + XS1;      // [2*D] LayerNorm gamma, beta of the next normalising phase
+  float* attp = lnp + 2 * D;   // [ATTP]
+  float* part = attp + ATTP;   // [PART]
+  float* qkv_s = part + PART;  // [3*HS]
+  float* pubA = qkv_s + 3 * HS;   // [PA::CPW] finished c_attn columns
+  float* pubC = pubA + PA::CPW;   // [PC::CPW] residual stream after the attention projection
+  float* pubD = pubC + PC::CPW;   // [PD::CPW] finished c_fc columns
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
   if (tid == 0) sh.bail = 0;
-  for (int e = tid; e < XS; e += NT) xs[e] = 0.f;
-  __syncthreads();
+  for (int e = tid; e < XS0 + XS1; e += NT) lds[e] = 0.f;  // the padding of xs0 beyond D stays zero for good
 
-  // items of this workgroup per phase (fewer than ITEMS only when N is not a multiple of G*CPW)
-  auto items_of = [&](int N, int CPW, int S) {
-    int n = N - wg * CPW;
-    n = n > CPW ? CPW : (n < 0 ? 0 : n);
-    return n * S;
+  // columns this workgroup finishes per phase (fewer than CPW only at the ragged end)
+  auto cols_of = [&](int N, int CPW) {
+    const int n = N - wg * CPW;
+    return n > CPW ? CPW : (n < 0 ? 0 : n);
   };
-  const int nitA = items_of(PA::N, PA::CPW, PA::S), nitC = items_of(PC::N, PC::CPW, PC::S);
-  const int nitD = items_of(PD::N, PD::CPW, PD::S), nitE = items_of(PE::N, PE::CPW, PE::S);
+  const int ncA = cols_of(PA::N, PA::CPW), ncC = cols_of(PC::N, PC::CPW);
+  const int ncD = cols_of(PD::N, PD::CPW), ncE = cols_of(PE::N, PE::CPW);
+  // local column this lane finishes (lane cc of wave v: column v + cc * NW)
+  const int fc = wave + lane * NW;
+  const bool finA = lane < PA::CW && fc < ncA, finC = lane < PC::CW && fc < ncC, finD = lane < PD::CW && fc < ncD;
 
   // attention role: head and slice of the positions; threads form 32 key groups
   // (tid >> 4) of 16 lanes (tid & 15)
@@ -436,21 +524,29 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   const int ah = wg / SPLIT, as = wg - ah * SPLIT;
 
   const LayerParamOffsets po = layer_param_offsets(D);
-  WSet<MAXI, C::SD, C::I8> ws;
-  typedef typename std::conditional<C::I8, int, float4>::type Item;
+  typedef WSet<MAXI, I8> WS;
+  WS ws0, ws1;
+  WS& wX = ws0;                // c_attn, c_fc
+  WS& wY = DUAL ? ws1 : ws0;   // attention c_proj, mlp c_proj
+  float4 lnreg[NLN];
+  typedef typename std::conditional<I8, int, float4>::type Item;
   const Item* slabs = reinterpret_cast<const Item*>(a.slabs);
   float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
   int tok = a.tok[0];
 
-  load_items<PA>(ws, slabs, a.lparams + po.bA, a.lparams + po.sA, nitA, wg, wave, lane);
-  load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
+  load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+  // FOLD: only the final LayerNorm has parameters, and they stay in lnp for good
+  if (FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
+  else request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
+  deposit_ln<D>(lnreg, lnp);
+  __syncthreads();
 
   for (int step = 0; step < a.nsteps; ++step) {
     const int pos = a.pos0 + step;
     TRACE(0);
     // ---- embedding: every workgroup builds the row itself (instructions.js:795-821) ----
-    for (int e = tid; e < D; e += NT) xs[e] = a.wte[(size_t)tok * D + e] + a.wpe[(size_t)pos * D + e];
+    for (int e = tid; e < D; e += NT) xs0[e] = a.wte[(size_t)tok * D + e] + a.wpe[(size_t)pos * D + e];
     __syncthreads();
 
     // slice of positions 0..pos for the attention role
@@ -462,7 +558,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     const bool has_new = pos >= c0 && pos < c1;  // this slice holds the new position
     const int nkv = c1 > c0 ? (c1 - c0 + 31) / 32 : 0;  // key batches of this slice
 
-    float own_r = 0.f;  // residual stream value of the column this thread finishes in the d-wide phases
+    float own_r = 0.f;  // residual stream value of the column this lane finishes in the attention projection
 
     for (int li = 0; li < a.L; ++li) {
       const Item* slab = slabs + (size_t)li * a.slab_stride;
@@ -474,21 +570,23 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       {
         constexpr int PH = PH_QKV;
         if (li > 0) {
-          poll_words<D>(a.bufR2, ep, xs, a.err);
+          poll_words<D>(a.bufR2, ep, xs0, a.err);
+          if (!FOLD) deposit_ln<D>(lnreg, lnp);
           __syncthreads();
           if (sh.bail) return;
         }
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        own_r = (tid < PC::CPW && wg * PC::CPW + tid < D) ? xs[wg * PC::CPW + tid] : 0.f;
-        gemv_items<PA, true>(ws, xs, part, nitA, wave, lane);
+        if (DUAL) load_items<PC>(wY, slab + a.slab_offC, lp + po.bC, lp + po.sC, ncC, wg, wave, lane);
+        own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
+        const float dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane);
         TRACE5(2);
+        if (finA) pubA[fc] = finish<I8>(dot, wX);
         __syncthreads();
         ++ep;
-        if (tid < PA::CPW && wg * PA::CPW + tid < PA::N)
-          publish(a.bufQKV + wg * PA::CPW + tid, colval<PA, C::I8>(part, tid, ws), ep);
+        if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
         TRACE5(4);
-        load_items<PC>(ws, slab + a.slab_offC, lp + po.bC, lp + po.sC, nitC, wg, wave, lane);
+        if (!DUAL) load_items<PC>(wY, slab + a.slab_offC, lp + po.bC, lp + po.sC, ncC, wg, wave, lane);
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -602,6 +700,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
+        if (DUAL) {
+          load_items<PD>(wX, slab + a.slab_offD, lp + po.bD, lp + po.sD, ncD, wg, wave, lane);
+          if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
+        }
         // merge of the slices of each head (flash-decoding): element e of head h is
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
         // derives the weights of its head itself (broadcast LDS reads, no barrier)
@@ -625,73 +727,82 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
               Lsum += phd[s2 * (HS + 2) + HS + 1] * wv;
               val += phd[s2 * (HS + 2) + c] * wv;
             }
-            xs[e] = val * fast_rcp(Lsum);
+            xs1[e] = val * fast_rcp(Lsum);
           }
+        }
+        if (XS0 > D) {  // the hidden row of the layer before reached into the padding
+          for (int e = D + tid; e < XS0; e += NT) xs1[e] = 0.f;
         }
         __syncthreads();
         TRACE5(1);
-        gemv_items<PC, false>(ws, xs, part, nitC, wave, lane);
+        const float dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
         TRACE5(2);
+        if (finC) pubC[fc] = own_r + finish<I8>(dot, wY);  // model.js:159
         __syncthreads();
         ++ep;
-        if (tid < PC::CPW && wg * PC::CPW + tid < D) {
-          own_r += colval<PC, C::I8>(part, tid, ws);  // model.js:159
-          publish(a.bufR1 + wg * PC::CPW + tid, own_r, ep);
-        }
+        if (tid < ncC) publish(a.bufR1 + wg * PC::CPW + tid, pubC[tid], ep);
         TRACE5(4);
-        load_items<PD>(ws, slab + a.slab_offD, lp + po.bD, lp + po.sD, nitD, wg, wave, lane);
-        load_ln<D>(ws, lp + po.ln2g, lp + po.ln2b, lane);
+        if (!DUAL) {
+          load_items<PD>(wX, slab + a.slab_offD, lp + po.bD, lp + po.sD, ncD, wg, wave, lane);
+          if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
+        }
         TRACE5(5);
       }
 
       // ======================= c_fc: LN2 + fc + GELU =======================
       {
         constexpr int PH = PH_FC;
-        poll_words<D>(a.bufR1, ep, xs, a.err);
+        poll_words<D>(a.bufR1, ep, xs0, a.err);
+        if (!FOLD) deposit_ln<D>(lnreg, lnp);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        gemv_items<PD, true>(ws, xs, part, nitD, wave, lane);
+        if (DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
+        const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane);
         TRACE5(2);
+        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, wX));  // model.js:188
         __syncthreads();
         ++ep;
-        if (tid < PD::CPW && wg * PD::CPW + tid < HID)
-          publish(a.bufH + wg * PD::CPW + tid, gelu_ref(colval<PD, C::I8>(part, tid, ws)), ep);  // model.js:188
+        if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
         TRACE5(4);
-        load_items<PE>(ws, slab + a.slab_offE, lp + po.bE, lp + po.sE, nitE, wg, wave, lane);
+        if (!DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
         TRACE5(5);
       }
 
       // ======================= mlp c_proj: fc2 + residual =======================
       {
         constexpr int PH = PH_FC2;
-        poll_words<HID>(a.bufH, ep, xs, a.err);
+        // weights of the phase after this one: the next layer's c_attn share with its
+        // LayerNorm; after the last layer the final LayerNorm (and, with two register
+        // sets, already the first layer's share for the next token)
+        auto request_next = [&]() {
+          if (li + 1 < a.L) {
+            load_items<PA>(wX, slab + a.slab_stride, lp + po.stride + po.bA, lp + po.stride + po.sA, ncA, wg, wave, lane);
+            if (!FOLD) request_ln<D>(lnreg, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
+          } else {
+            if (!FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
+            if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+          }
+        };
+        poll_words<HID>(a.bufH, ep, xs1, a.err);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        gemv_items<PE, false>(ws, xs, part, nitE, wave, lane);
+        if (DUAL) request_next();
+        gemv_split<PE>(wY, xs1, part, ncE, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
-        if (tid < PC::CPW && wg * PC::CPW + tid < D)
-          publish(a.bufR2 + wg * PC::CPW + tid, own_r + colval<PE, C::I8>(part, tid, ws), ep);  // model.js:205
+        if (tid < ncE) publish(a.bufR2 + wg * PE::CPW + tid, pubC[tid] + finish<I8>(column_sum<PE>(part, tid), wY), ep);  // model.js:205
         TRACE5(4);
-        // next layer's c_attn share, or the first layer's for the next step
-        if (li + 1 < a.L) {
-          load_items<PA>(ws, slab + a.slab_stride, lp + po.stride + po.bA, lp + po.stride + po.sA, nitA, wg, wave, lane);
-          load_ln<D>(ws, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b, lane);
-        } else {
-          load_ln<D>(ws, a.lnf_g, a.lnf_b, lane);
-        }
+        if (!DUAL) request_next();
         TRACE5(5);
-        // xs beyond D must be zero again for the D-wide phases that follow
-        for (int e = D + tid; e < XS; e += NT) xs[e] = 0.f;
-        __syncthreads();
       }
     }
 
     // ======================= final LayerNorm + vocabulary projection =======================
-    poll_words<D>(a.bufR2, ep, xs, a.err);
+    poll_words<D>(a.bufR2, ep, xs0, a.err);
+    if (!FOLD) deposit_ln<D>(lnreg, lnp);
     __syncthreads();
     if (sh.bail) return;
     wait_loads();
@@ -704,31 +815,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       v1 = v1 > a.V ? a.V : v1;
       // final LayerNorm of the row, in registers (each wave for itself)
       float4 xv[S];
-      {
-        float sum = 0.f;
-#pragma unroll
-        for (int s2 = 0; s2 < S; ++s2) {
-          xv[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + lane * 4);
-          sum += (xv[s2].x + xv[s2].y) + (xv[s2].z + xv[s2].w);
-        }
-        const float mean = wave_sum(sum) * (1.0f / (float)D);
-        float q = 0.f;
-#pragma unroll
-        for (int s2 = 0; s2 < S; ++s2) {
-          const bool in = s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D;
-          xv[s2].x -= mean; xv[s2].y -= mean; xv[s2].z -= mean; xv[s2].w -= mean;
-          const float qq = (xv[s2].x * xv[s2].x + xv[s2].y * xv[s2].y) + (xv[s2].z * xv[s2].z + xv[s2].w * xv[s2].w);
-          q += in ? qq : 0.f;
-        }
-        const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)D) + 1e-5f);
-#pragma unroll
-        for (int s2 = 0; s2 < S; ++s2) {
-          xv[s2].x = ws.g[s2].x * (xv[s2].x * rstd) + ws.b[s2].x;
-          xv[s2].y = ws.g[s2].y * (xv[s2].y * rstd) + ws.b[s2].y;
-          xv[s2].z = ws.g[s2].z * (xv[s2].z * rstd) + ws.b[s2].z;
-          xv[s2].w = ws.g[s2].w * (xv[s2].w * rstd) + ws.b[s2].w;
-        }
-      }
+      input_row<D, true, true>(xv, xs0, lnp, lane);
       float best = -INFINITY;
       int besti = 0x7fffffff;
       for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
@@ -780,11 +867,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
     TRACE(2 + a.L * 8);
     if (step + 1 < a.nsteps) {
-      load_items<PA>(ws, slabs, a.lparams + po.bA, a.lparams + po.sA, nitA, wg, wave, lane);
-      load_ln<D>(ws, a.lparams + po.ln1g, a.lparams + po.ln1b, lane);
+      if (!DUAL) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+      if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
     poll_words<2 * C::G>(a.bufAM, ep, attp, a.err);
+    if (!FOLD && step + 1 < a.nsteps) deposit_ln<D>(lnreg, lnp);  // every wave is past the final LayerNorm: the arg-max words need all of them
     __syncthreads();
     if (sh.bail) return;
     TRACE(3 + a.L * 8);
@@ -815,8 +903,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   }
 }
 
+// rowscale (may be null): the gamma of the LayerNorm in front of the matrix, folded in as
+// diag(gamma) W.
 __global__ void build_slab_kernel(const float* __restrict__ W, int ldw, int K, int N, int cpw, int S, size_t total,
-                                  float4* __restrict__ slab) {
+                                  const float* __restrict__ rowscale, float4* __restrict__ slab) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int lane = (int)(idx & 63);
@@ -828,8 +918,19 @@ __global__ void build_slab_kernel(const float* __restrict__ W, int ldw, int K, i
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (col < N)
     for (int e = 0; e < 4; ++e)
-      if (k + e < K) v[e] = W[(size_t)(k + e) * ldw + col];
+      if (k + e < K) v[e] = W[(size_t)(k + e) * ldw + col] * (rowscale ? rowscale[k + e] : 1.0f);
   slab[idx] = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// out[n] = bias[n] + sum_k beta[k] W[k][n]: the beta of the LayerNorm in front of the
+// matrix, folded into the bias (accumulated in double, rounded once).
+__global__ void fold_ln_bias_kernel(const float* __restrict__ W, int ldw, int K, int N, const float* __restrict__ beta,
+                                    const float* __restrict__ bias, float* __restrict__ out) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  double acc = 0.0;
+  for (int k = 0; k < K; ++k) acc += (double)beta[k] * (double)W[(size_t)k * ldw + n];
+  out[n] = (float)((double)bias[n] + acc);
 }
 
 // int8: item (w, j = c*S + seg, lane) is one word holding rows k..k+3 (k = seg*256 + lane*4)
@@ -858,11 +959,10 @@ __global__ void build_slab_i8_kernel(const int32_t* __restrict__ Wq, int ldwq, i
 template <class C>
 size_t lds_bytes_of() {
   typedef Phases<C> PS;
-  constexpr int XS = C::SH * SEG;
+  constexpr int XS = (C::SD + C::SH) * SEG;
   constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;
-  constexpr int CPWMAX = PS::A::CPW > PS::Dd::CPW ? PS::A::CPW : PS::Dd::CPW;
-  constexpr int PART = 32 * (C::HS + 4) > CPWMAX * NW ? 32 * (C::HS + 4) : CPWMAX * NW;
-  const size_t need = sizeof(float) * (size_t)(XS + ATTP + PART + 3 * C::HS + C::H * C::SPLIT + 16);
+  constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
+  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + PS::Cc::CPW + PS::Dd::CPW + 16);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
   const size_t one_per_cu = 84 * 1024;
   return need > one_per_cu ? need : one_per_cu;
@@ -895,9 +995,14 @@ PhaseGeom make_geom(int N, int K) {
 
 size_t slab_float4s(const PhaseGeom& g) { return (size_t)PD_GRID * g.cpw * g.S * 64; }
 
-hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, float4* slab, hipStream_t s) {
+hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const float* rowscale, float4* slab, hipStream_t s) {
   const size_t total = slab_float4s(g);
-  build_slab_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(W, ldw, K, g.N, g.cpw, g.S, total, slab);
+  build_slab_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(W, ldw, K, g.N, g.cpw, g.S, total, rowscale, slab);
+  return hipGetLastError();
+}
+
+hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* beta, const float* bias, float* out, hipStream_t s) {
+  fold_ln_bias_kernel<<<(unsigned)((N + 127) / 128), 128, 0, s>>>(W, ldw, K, N, beta, bias, out);
   return hipGetLastError();
 }
 

@@ -223,10 +223,11 @@ static int setup_persistent(Model* m) {
       LAUNCH(build_slab_i8(l.fc2.q, d / 4, hid, gE, sl + a.slab_offE, rt().stream));
     } else {
       float4* sl = (float4*)slb;
-      LAUNCH(build_slab(l.attn.w, 3 * d, d, gA, sl, rt().stream));
-      LAUNCH(build_slab(l.proj.w, d, d, gC, sl + a.slab_offC, rt().stream));
-      LAUNCH(build_slab(l.fc.w, hid, d, gD, sl + a.slab_offD, rt().stream));
-      LAUNCH(build_slab(l.fc2.w, d, hid, gE, sl + a.slab_offE, rt().stream));
+      // the two LayerNorms go into the matrices they feed: diag(gamma) W here, beta W into the bias below
+      LAUNCH(build_slab(l.attn.w, 3 * d, d, gA, l.ln1_g, sl, rt().stream));
+      LAUNCH(build_slab(l.proj.w, d, d, gC, nullptr, sl + a.slab_offC, rt().stream));
+      LAUNCH(build_slab(l.fc.w, hid, d, gD, l.ln2_g, sl + a.slab_offD, rt().stream));
+      LAUNCH(build_slab(l.fc2.w, d, hid, gE, nullptr, sl + a.slab_offE, rt().stream));
     }
     float* lp = lparams + (size_t)i * po.stride;
     const struct { int off; const float* src; int n; } parts[12] = {
@@ -235,6 +236,10 @@ static int setup_persistent(Model* m) {
         {po.sA, l.attn.s, 3 * d}, {po.sC, l.proj.s, d}, {po.sD, l.fc.s, hid}, {po.sE, l.fc2.s, d}};
     for (const auto& pt : parts)
       if (pt.src) WGPT_HIP(hipMemcpyAsync(lp + pt.off, pt.src, sizeof(float) * pt.n, hipMemcpyDeviceToDevice, rt().stream));
+    if (!i8) {
+      LAUNCH(fold_ln_bias(l.attn.w, 3 * d, d, 3 * d, l.ln1_b, l.attn_b, lp + po.bA, rt().stream));
+      LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_b, l.fc_b, lp + po.bD, rt().stream));
+    }
   }
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   a.slabs = slabs;
