@@ -57,6 +57,11 @@ struct PersistentArgs {
   int32_t* out_tok;    // [nsteps] arg-max of each step
   int* err;            // set non-zero when a bounded wait expired
   unsigned long long* trace;  // optional [G][512] clock samples of the last step (WGPT_TRACE builds), or null
+  // naps (about 64 clocks each) between a publish and the first poll of the words that
+  // follow it: [0] residual row into c_attn, [1] q/k/v into the attention slices,
+  // [2] attention outputs on the attention workgroups, [3] on the others,
+  // [4] residual row into c_fc, [5] hidden row, [6] arg-max candidates
+  int delay[7];
   unsigned ebase;      // epoch of the last word published by earlier launches
   int pos0, nsteps;
 };

@@ -179,11 +179,13 @@ struct Phase {
   static constexpr bool RAGGED = CPW * PD_GRID != N;       // some workgroups finish fewer than CPW columns
 };
 
-#ifndef WGPT_POLL_DELAY
-#define WGPT_POLL_DELAY 0
-#endif
+// Idles the wave for about 64 * units clocks.
+__device__ __forceinline__ void nap(int units) {
+  for (int i = 0; i < units; ++i) __builtin_amdgcn_s_sleep(1);
+}
+
 template <int N>
-__device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err) {
+__device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err, int delay) {
   constexpr int NP = (N + NT - 1) / NT;
   const int t = opaque(threadIdx.x);
   unsigned pending = 0;
@@ -191,9 +193,7 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
   for (int i = 0; i < NP; ++i)
     if (i * NT + NT <= N || t + i * NT < N) pending |= 1u << i;
   unsigned spins = 0;
-#if WGPT_POLL_DELAY > 0
-  __builtin_amdgcn_s_sleep(WGPT_POLL_DELAY);
-#endif
+  nap(delay);
   while (pending) {
     u64 pk[NP];
 #pragma unroll
@@ -333,7 +333,11 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
     float sum = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
+#ifdef WGPT_DBG_NOSTATS
+    const float mean = sum * 1e-30f;
+#else
     const float mean = wave_sum(sum) * (1.0f / (float)K);
+#endif
     float q = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
@@ -343,7 +347,11 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
       const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
       q += in ? qq : 0.f;
     }
+#ifdef WGPT_DBG_NOSTATS
+    const float rstd = 1.0f + q * 1e-30f;
+#else
     const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)K) + 1e-5f);
+#endif
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
       const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
@@ -570,7 +578,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       {
         constexpr int PH = PH_QKV;
         if (li > 0) {
-          poll_words<D>(a.bufR2, ep, xs0, a.err);
+          poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0]);
           if (!FOLD) deposit_ln<D>(lnreg, lnp);
           __syncthreads();
           if (sh.bail) return;
@@ -617,6 +625,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         {
           unsigned pending = tid < 3 * HS ? 1u : 0u;
           unsigned spins = 0;
+          nap(a.delay[1]);
           const int which = tid / HS, e = tid - which * HS;
           const u64* src = a.bufQKV + which * D + ah * HS + e;
           while (pending) {
@@ -696,7 +705,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
         constexpr int PH = PH_PROJ;
-        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err);
+        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3]);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -752,7 +761,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= c_fc: LN2 + fc + GELU =======================
       {
         constexpr int PH = PH_FC;
-        poll_words<D>(a.bufR1, ep, xs0, a.err);
+        poll_words<D>(a.bufR1, ep, xs0, a.err, a.delay[4]);
         if (!FOLD) deposit_ln<D>(lnreg, lnp);
         __syncthreads();
         wait_loads();
@@ -760,7 +769,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
         const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane);
         TRACE5(2);
-        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, wX));  // model.js:188
+        if (finD) 
+#ifdef WGPT_DBG_NOGELU
+          pubD[fc] = finish<I8>(dot, wX) * 0.01f;
+#else
+          pubD[fc] = gelu_ref(finish<I8>(dot, wX));
+#endif
+  // model.js:188
         __syncthreads();
         ++ep;
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
@@ -784,7 +799,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
             if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
           }
         };
-        poll_words<HID>(a.bufH, ep, xs1, a.err);
+        poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5]);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -801,7 +816,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
 
     // ======================= final LayerNorm + vocabulary projection =======================
-    poll_words<D>(a.bufR2, ep, xs0, a.err);
+    poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0]);
     if (!FOLD) deposit_ln<D>(lnreg, lnp);
     __syncthreads();
     if (sh.bail) return;
@@ -871,7 +886,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
-    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err);
+    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err, a.delay[6]);
     if (!FOLD && step + 1 < a.nsteps) deposit_ln<D>(lnreg, lnp);  // every wave is past the final LayerNorm: the arg-max words need all of them
     __syncthreads();
     if (sh.bail) return;

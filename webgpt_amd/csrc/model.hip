@@ -262,6 +262,22 @@ static int setup_persistent(Model* m) {
   a.tok = m->tok_dev;
   a.out_tok = m->out_tok_dev;
   a.err = m->perr;
+  {
+    // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
+    // curves are flat within a few percent around them and over context length);
+    // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
+    static const int tuned[4][7] = {{16, 4, 28, 96, 24, 20, 40},    // d <= 768
+                                    {20, 0, 48, 96, 28, 32, 64},    // d = 1024
+                                    {20, 0, 48, 96, 4, 20, 40},     // d = 1280
+                                    {40, 0, 48, 96, 32, 40, 40}};   // d = 1600, int8
+    const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : 3];
+    for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
+    if (const char* e = getenv("WEBGPT_AMD_POLL_DELAYS")) {
+      int v[7];
+      if (sscanf(e, "%d,%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6]) == 7)
+        for (int i = 0; i < 7; ++i) a.delay[i] = v[i] < 0 ? 0 : (v[i] > 1024 ? 1024 : v[i]);
+    }
+  }
   a.trace = nullptr;
 #ifdef WGPT_TRACE
   // Profiling builds: per-workgroup clock samples of the last step of each launch.
