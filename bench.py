@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--mode", type=int, default=None, help="decode implementation (default: library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="first run three 256 MiB device-to-device copies (a kernel of known traffic, for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (batch-1 decode does not shard usefully); "
@@ -67,6 +70,16 @@ def main():
     if cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
         print(f"bench.py: prompt {cfg['prompt']} + warmup + steps exceeds n_ctx {cfg['n_ctx']}", file=sys.stderr)
         sys.exit(2)
+    if args.copy_probe:
+        from webgpt_amd import _lib, blocks
+        blocks.Device(0)
+        n = 256 << 20
+        src, dst = blocks.Buffer([n // 4]), blocks.Buffer([n // 4])
+        for _ in range(3):
+            _lib.call("wgpt_copy", dst.handle, 0, src.handle, 0, n)
+        _lib.call("wgpt_sync")
+        src.destroy()
+        dst.destroy()
     tensors = dict(synth.make_tensors(cfg, args.seed))
     prompt = synth.make_prompt(cfg, args.seed)
     gpt = GPT(None, "bpe", tensors=tensors, params=synth.model_params(cfg))
@@ -117,7 +130,7 @@ def main():
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
     # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)
-    traffic = 523.5e6 if (persistent and args.config == "gpt2-117m") else None
+    traffic = 519.0e6 if (persistent and args.config == "gpt2-117m") else None
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
