@@ -262,11 +262,14 @@ __global__ __launch_bounds__(WG) void gemm_tile64(int M, int N, int K, const flo
 // FastMatMulBlock as a dense contraction on the matrix cores (prefill, M >= 16):
 // C = epi(A . W + bias). fp32 MFMA v_mfma_f32_32x32x2_f32: per instruction a wave
 // multiplies a 32x2 slice of A by a 2x32 slice of W into a 32x32 fp32 accumulator
-// (16 VGPRs per lane). Workgroup tile TM x 64 (TM = 64 or 128), four waves in a 2x2
-// arrangement, each owning (TM/2) x 32 of C; K advances in steps of 16 through LDS
-// with the next step's global loads held in registers while the current one is
-// multiplied. A is staged as [m][k] with a row stride of 17 floats (lanes of an
-// A-operand read hit distinct banks), W as [k][n].
+// (16 VGPRs per lane). Workgroup tile TM x TN (64 or 128 each), four waves in a 2x2
+// arrangement, each owning (TM/2) x (TN/2) of C as RB x CB accumulator blocks, so an
+// operand fragment read from LDS feeds CB (or RB) instructions. K advances in steps
+// of BK = 32 through two LDS stages: the next step's global loads are in flight while
+// the current one is multiplied and land in the other stage (one barrier per step).
+// A is staged as [m][BK + 4] with the k of a step permuted to (k odd, k / 2), so the
+// values a lane feeds to four consecutive instructions are one 128-bit read; W as
+// [k][n].
 // Operand lane mapping of the instruction: lane l supplies A[row l%32][k l/32] and
 // W[k l/32][col l%32]; accumulator register r of lane l is
 // C[row (r/4)*8 + (l/32)*4 + r%4][col l%32].
@@ -275,77 +278,112 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // With kchunk < K (split-K) slice blockIdx.z covers k in [z*kchunk, (z+1)*kchunk) and
 // writes its raw partial sums to C + z*M*ldc (bias, epilogue: gemv_reduce afterwards).
-template <int TM>
+template <int TM, int TN, int BK>
 __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
                                                  const float* __restrict__ W, int ldw, const float* __restrict__ bias,
                                                  float* C, int ldc, int epi, const float* resid) {
-  constexpr int BK = 16, TN = 64, AST = BK + 1;
-  constexpr int RB = TM / 64;  // 32-row blocks per wave
-  __shared__ float As[TM * AST];
-  __shared__ float Bs[BK * TN];
+  constexpr int AST = BK + 4;                // floats per staged A row (16-byte aligned, odd multiple of 4 banks)
+  constexpr int RB = TM / 64, CB = TN / 64;  // 32x32 accumulator blocks per wave
+  constexpr int KQ = BK / 4;                 // float4 per A row of a step
+  constexpr int AROWS = WG / KQ;             // A rows covered by one pass of the workgroup
+  constexpr int NA = TM / AROWS;             // float4 per thread of the A tile of a step
+  constexpr int BROWS = WG / (TN / 4);       // W rows covered by one pass of the workgroup
+  constexpr int NB = BK / BROWS;             // float4 per thread of the W tile of a step
+  constexpr int HK = BK / 2;                 // MFMA instructions per step and accumulator block
+  __shared__ __attribute__((aligned(16))) float As[2][TM * AST];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * TN];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
-  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * 32;
-  // global -> register staging: A tile TM x 16 (float4 along k), W tile 16 x 64 (float4 along n)
-  const int arow = tid >> 2, akq = (tid & 3) * 4;
-  const int brow = tid >> 4, bnq = (tid & 15) * 4;
-  float4 ga[RB], gb;
+  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
+  const int arow = tid / KQ, akq = (tid % KQ) * 4;
+  const int brow = tid / (TN / 4), bnq = (tid % (TN / 4)) * 4;
+  float4 ga[NA], gb[NB];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      const int m = m0 + arow + r * 64;
+    for (int r = 0; r < NA; ++r) {
+      const int m = m0 + arow + r * AROWS;
       ga[r] = (m < M && k0 + akq < K) ? ld4(A + (size_t)m * lda + k0 + akq) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    gb = (k0 + brow < K && n0 + bnq < N) ? ld4(W + (size_t)(k0 + brow) * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
-  };
-  auto stage = [&]() {
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      float* d = As + (arow + r * 64) * AST + akq;
-      d[0] = ga[r].x; d[1] = ga[r].y; d[2] = ga[r].z; d[3] = ga[r].w;
+    for (int r = 0; r < NB; ++r) {
+      const int k = k0 + brow + r * BROWS;
+      gb[r] = (k < K && n0 + bnq < N) ? ld4(W + (size_t)k * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    st4(Bs + brow * TN + bnq, gb);
   };
-  f32x16 acc[RB];
+  auto stage = [&](int st) {
+#pragma unroll
+    for (int r = 0; r < NA; ++r) {
+      // k = akq + j goes to slot (k & 1) * HK + k / 2: (x, z) are the even k, (y, w) the odd
+      float* d = As[st] + (arow + r * AROWS) * AST + (akq >> 1);
+      *reinterpret_cast<float2*>(d) = make_float2(ga[r].x, ga[r].z);
+      *reinterpret_cast<float2*>(d + HK) = make_float2(ga[r].y, ga[r].w);
+    }
+#pragma unroll
+    for (int r = 0; r < NB; ++r) st4(Bs[st] + (brow + r * BROWS) * TN + bnq, gb[r]);
+  };
+  f32x16 acc[RB][CB];
 #pragma unroll
   for (int r = 0; r < RB; ++r)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
+    for (int c = 0; c < CB; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[r][c][i] = 0.f;
 
   const int kbeg = blockIdx.z * kchunk;
   const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
   C += (size_t)blockIdx.z * M * ldc;
   K = kend;
   fetch(kbeg);
+  stage(0);
+  __syncthreads();
+  int st = 0;
+  const int h = lane >> 5, l32 = lane & 31;
   for (int k0 = kbeg; k0 < kend; k0 += BK) {
-    stage();
-    __syncthreads();
-    if (k0 + BK < kend) fetch(k0 + BK);
-    const float* ap = As + (wm + (lane & 31)) * AST + (lane >> 5);
-    const float* bp = Bs + (lane >> 5) * TN + wn + (lane & 31);
+    const bool more = k0 + BK < kend;
+    if (more) fetch(k0 + BK);
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      const float b = bp[kk * TN];
+    for (int q = 0; q < HK / 4; ++q) {  // four instructions per block and quarter-step: one 128-bit A read each
+      float av[RB][4], bv[CB][4];
 #pragma unroll
-      for (int r = 0; r < RB; ++r) acc[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[r * 32 * AST + kk], b, acc[r], 0, 0, 0);
-    }
-    __syncthreads();
-  }
-  const int n = n0 + wn + (lane & 31);
-  if (n >= N) return;
-  const float bv = bias ? bias[n] : 0.f;
-#pragma unroll
-  for (int r = 0; r < RB; ++r)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int m = m0 + wm + r * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-      if (m < M) {
-        float v = acc[r][i] + bv;
-        if (epi == EPI_GELU) v = gelu_ref(v);
-        else if (epi == EPI_RESIDUAL) v += resid[(size_t)m * ldc + n];
-        C[(size_t)m * ldc + n] = v;
+      for (int r = 0; r < RB; ++r) {
+        const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + q * 4);
+        av[r][0] = v.x; av[r][1] = v.y; av[r][2] = v.z; av[r][3] = v.w;
       }
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        const float* bp = Bs[st] + (h + 8 * q) * TN + wn + c * 32 + l32;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[c][i] = bp[2 * i * TN];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+          for (int c = 0; c < CB; ++c) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[r][i], bv[c][i], acc[r][c], 0, 0, 0);
     }
+    if (more) stage(st ^ 1);
+    __syncthreads();
+    st ^= 1;
+  }
+#pragma unroll
+  for (int c = 0; c < CB; ++c) {
+    const int n = n0 + wn + c * 32 + l32;
+    if (n >= N) continue;
+    const float bvs = bias ? bias[n] : 0.f;
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm + r * 32 + (i >> 2) * 8 + h * 4 + (i & 3);
+        if (m < M) {
+          float v = acc[r][c][i] + bvs;
+          if (epi == EPI_GELU) v = gelu_ref(v);
+          else if (epi == EPI_RESIDUAL) v += resid[(size_t)m * ldc + n];
+          C[(size_t)m * ldc + n] = v;
+        }
+      }
+  }
 }
 
 // ResidualBlock, instructions.js:381-382
@@ -719,27 +757,39 @@ hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const fl
 
 size_t gemm_workspace_floats(int M, int N) { return (size_t)8 * M * N; }
 
+namespace {
+template <int TM, int TN, int BK>
+void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const float* W, int ldw, const float* bias, float* C,
+                   int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  const dim3 grid(cdiv(N, TN), cdiv(M, TM), S);
+  if (S == 1) {
+    gemm_mfma<TM, TN, BK><<<grid, WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+  } else {
+    // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
+    const int kchunk = (int)cdiv(cdiv(K, S), BK) * BK;
+    gemm_mfma<TM, TN, BK><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
+    gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  }
+}
+}  // namespace
+
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
                        float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
   if (M < 16) {
     // too few rows for a matrix-core tile: scalar-FMA tile kernel
     gemm_tile64<<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
-  } else if ((size_t)cdiv(N, 64) * cdiv(M, 128) >= 512) {
-    gemm_mfma<128><<<dim3(cdiv(N, 64), cdiv(M, 128)), WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
-  } else {
-    // few tiles: split K so that every compute unit gets work; partial sums are
-    // combined in ascending order by gemv_reduce (deterministic), bias last
-    const unsigned tiles = cdiv(N, 64) * cdiv(M, 64);
-    int S = 1;
-    while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
-    if (S == 1) {
-      gemm_mfma<64><<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
-    } else {
-      const int kchunk = (int)cdiv(cdiv(K, S), 16) * 16;
-      gemm_mfma<64><<<dim3(cdiv(N, 64), cdiv(M, 64), S), WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
-      gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
-    }
+    return hipGetLastError();
   }
+  // 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
+  // best or within 3 % of it from 128 to 1024 rows); then split K (at most 8 ways, slices of
+  // at least 128) until there are two workgroups per compute unit.
+  const bool big = (size_t)cdiv(M, 128) * cdiv(N, 128) >= 512;
+  const int t = big ? 128 : 64;
+  int S = 1;
+  const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
+  while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
+  if (big) run_gemm_mfma<128, 128, 32>(M, N, K, S, A, lda, W, ldw, bias, C, ldc, epi, resid, workspace, s);
+  else run_gemm_mfma<64, 64, 32>(M, N, K, S, A, lda, W, ldw, bias, C, ldc, epi, resid, workspace, s);
   return hipGetLastError();
 }
 
