@@ -178,7 +178,7 @@ class GPT {
     const int8 = names.some((n) => n.endsWith(".weight.q"));
     const handle = native.modelCreate(params.n_layer, params.n_head, params.n_embd, params.n_ctx, params.vocab_size, int8 ? 1 : 0, params.max_prefill || 0, this._flags);
     for (const name of names) {
-      const data = this._tensors ? this._tensors[name] : this.fetchBin(path.join(folder, `${name}_gpt.bin`));
+      const data = this._tensors ? this._tensors[name] : this.readTensor(folder, name, params);
       native.modelSetTensor(handle, name, data);
     }
     native.modelFinalize(handle);
@@ -208,6 +208,34 @@ class GPT {
         "ln_2.weight", "ln_2.bias", "mlp.c_fc.weight", "mlp.c_fc.bias", "mlp.c_proj.weight", "mlp.c_proj.bias"]) names.push(`transformer.h.${i}.${s}`);
     }
     return names.concat(["transformer.ln_f.weight", "transformer.ln_f.bias"]);
+  }
+
+  // Shape of a tensor file as the forward path wants it: linear weights [in, out], the layout
+  // other/conversion_scripts/*.py write for HF GPT-2 Conv1D modules (model.js:404-417).
+  tensorShape(name, params) {
+    const d = params.n_embd;
+    const linear = { "attn.c_attn.weight": [1, 3], "attn.c_proj.weight": [1, 1], "mlp.c_fc.weight": [1, 4], "mlp.c_proj.weight": [4, 1] };
+    if (name === "transformer.wte.weight") return [params.vocab_size, d];
+    if (name === "transformer.wpe.weight") return [params.n_ctx, d];
+    const rest = name.startsWith("transformer.h.") ? name.split(".").slice(3).join(".") : name;
+    if (linear[rest]) return [linear[rest][0] * d, linear[rest][1] * d];
+    const w = rest.replace(/\.bias$/, ".weight");
+    if (rest.endsWith(".bias") && linear[w]) return [linear[w][1] * d];
+    return [d];
+  }
+
+  // One <name>_gpt.bin. Two variations of the directory that earlier versions of the reference
+  // handled (condensed/condensed.js:1755-1783) are accepted through params_gpt.json:
+  // "bias": false - bias files are absent and read as zeros; "linear_layout": "out_in" - the four
+  // linear weights are stored [out, in] (torch nn.Linear, nanoGPT) and are transposed here.
+  readTensor(folder, name, params) {
+    const shape = this.tensorShape(name, params);
+    const count = shape.reduce((a, b) => a * b, 1);
+    if (name.endsWith(".bias") && params.bias === false) return G.zeros(count);
+    const data = this.fetchBin(path.join(folder, `${name}_gpt.bin`));
+    if (data.length !== count) throw new Error(`Model load failed: ${name}_gpt.bin holds ${data.length} values, expected ${count}.`);
+    if (shape.length === 2 && params.linear_layout === "out_in" && !name.startsWith("transformer.w")) return G.transpose(data, shape[1], shape[0]);
+    return data;
   }
 
   fetchBin(file) {

@@ -28,6 +28,45 @@ _FP = C.POINTER(C.c_float)
 _IP = C.POINTER(C.c_int32)
 
 
+_LINEAR = {"attn.c_attn.weight": (1, 3), "attn.c_proj.weight": (1, 1), "mlp.c_fc.weight": (1, 4), "mlp.c_proj.weight": (4, 1)}
+
+
+def tensor_shape(name, params):
+    """Shape of a tensor file of the weight directory as the forward path wants it
+    (linear weights [in, out], the layout other/conversion_scripts/*.py write for HF
+    GPT-2 `Conv1D` modules; model.js:404-417)."""
+    d = params["n_embd"]
+    if name == "transformer.wte.weight":
+        return (params["vocab_size"], d)
+    if name == "transformer.wpe.weight":
+        return (params["n_ctx"], d)
+    rest = name.split(".", 3)[3] if name.startswith("transformer.h.") else name
+    if rest in _LINEAR:
+        k, n = _LINEAR[rest]
+        return (k * d, n * d)
+    if rest.endswith(".bias") and rest[:-5] + ".weight" in _LINEAR:
+        return (_LINEAR[rest[:-5] + ".weight"][1] * d,)
+    return (d,)  # LayerNorm gains and biases
+
+
+def read_tensor(weightsFolder, name, params):
+    """One `<name>_gpt.bin` of little-endian f32 (model.js:484-488 `fetchBin`).
+    Two variations of the directory that earlier versions of the reference handled
+    (condensed/condensed.js:1755-1783) are accepted through params_gpt.json:
+    `"bias": false` - bias files are absent and read as zeros;
+    `"linear_layout": "out_in"` - the four linear weights are stored as torch
+    `nn.Linear` holds them, [out, in] (nanoGPT), and are transposed here."""
+    shape = tensor_shape(name, params)
+    if name.endswith(".bias") and not params.get("bias", True):
+        return np.zeros(shape, np.float32)
+    a = np.fromfile(os.path.join(weightsFolder, name + "_gpt.bin"), dtype="<f4")
+    if a.size != int(np.prod(shape)):
+        raise ValueError(f"Model load failed: {name}_gpt.bin holds {a.size} values, expected {int(np.prod(shape))}.")
+    if len(shape) == 2 and params.get("linear_layout", "in_out") == "out_in" and not name.startswith("transformer.w"):
+        return np.ascontiguousarray(a.reshape(shape[1], shape[0]).T)
+    return a.reshape(shape)
+
+
 class GPT:
     def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0):
         self.folder = folder
@@ -90,10 +129,10 @@ class GPT:
         params["bias"] = params.get("bias", True)
         return params
 
-    def _fetch(self, weightsFolder, name):
+    def _fetch(self, weightsFolder, name, params=None):
         if self._tensors is not None:
             return self._tensors[name]
-        return np.fromfile(os.path.join(weightsFolder, name + "_gpt.bin"), dtype="<f4")
+        return read_tensor(weightsFolder, name, params or self.params)
 
     def loadModel(self, folder):
         if self.initialized:
@@ -111,7 +150,7 @@ class GPT:
         if names is None:
             names = [n for n in self._directory_names(params)]
         for n in names:
-            a = np.ascontiguousarray(self._fetch(weightsFolder, n))
+            a = np.ascontiguousarray(self._fetch(weightsFolder, n, params))
             _lib.call("wgpt_model_set_tensor", self._handle, n.encode(), a.ctypes.data_as(C.c_void_p), a.nbytes)
         _lib.call("wgpt_model_finalize", self._handle)
         return {"handle": self._handle}, params
