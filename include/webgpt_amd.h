@@ -96,6 +96,12 @@ int wgpt_deembed(int d, int V, int T, wgpt_buf x, wgpt_buf wte, wgpt_buf logits)
 int wgpt_attention(int T, int d, float scale, int H, int hs, wgpt_buf x,
                    wgpt_buf Wq, wgpt_buf bq, wgpt_buf Wk, wgpt_buf bk, wgpt_buf Wv, wgpt_buf bv,
                    wgpt_buf Wo, wgpt_buf bo, wgpt_buf out);
+/* selectTopK + cpuSoftmax + sampleFromDistribution (globals.js:47-74) over a device
+ * buffer of V logits: *id receives the sampled index; ids[top_k] and probs[top_k]
+ * (either may be NULL) the selected indices (stable descending order: lowest index
+ * first among equal logits) and their float64 probabilities. top_k is clamped to V. */
+int wgpt_sample_topk(int V, int top_k, double temperature, double u, wgpt_buf logits, int32_t* id, int32_t* ids,
+                     double* probs);
 
 /* ---- whole model: GPT.loadModel + GPT.run (model.js:104-268, 270-488) ---- */
 typedef struct {
@@ -137,6 +143,13 @@ int wgpt_decode(wgpt_model m, int32_t token, float* logits);
  * selectTopK with top_k = 1, globals.js:66-74). out_tokens[steps] receives the
  * chosen ids; logits (may be NULL) the logits of the last step. */
 int wgpt_decode_greedy(wgpt_model m, int32_t token, int steps, int32_t* out_tokens, float* logits);
+/* Sampled continuation on the device: like wgpt_decode_greedy, but each step picks
+ * its token the way GPT.generate does (model.js:81-85): selectTopK(logits, top_k),
+ * cpuSoftmax(., temperature) in float64 and sampleFromDistribution (globals.js:47-74),
+ * with u[i] in [0,1) standing for the i-th Math.random() draw. The V logits never
+ * leave the device. top_k in [1, 1024], temperature > 0. */
+int wgpt_decode_sample(wgpt_model m, int32_t token, int steps, int top_k, double temperature, const double* u,
+                       int32_t* out_tokens, float* logits);
 int wgpt_model_reset_cache(wgpt_model m);
 int wgpt_model_position(wgpt_model m, int* pos);
 /* Activation taps of the last wgpt_prefill (needs WGPT_FLAG_TAPS): names follow

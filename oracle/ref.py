@@ -208,6 +208,18 @@ def dequantize_js(packed, absmax, count):
     return out
 
 
+def sample_topk(logits, top_k, temperature, u):
+    """(id, ids[k], probs[k]) of model.js:81-85 with `u` standing for Math.random()."""
+    logits = _f32(logits).ravel()
+    k = min(int(top_k), logits.size)
+    ids = np.empty(k, np.int32)
+    probs = np.empty(k, np.float64)
+    _lib.ref_sample_topk.restype = C.c_int
+    chosen = _lib.ref_sample_topk(logits.size, int(top_k), C.c_double(temperature), C.c_double(u), _fp(logits), _ip(ids),
+                                  probs.ctypes.data_as(C.POINTER(C.c_double)))
+    return int(chosen), ids, probs
+
+
 LAYER_F32 = ("ln1_g", "ln1_b", "attn_w", "attn_b", "proj_w", "proj_b", "ln2_g", "ln2_b", "fc_w", "fc_b", "fc2_w", "fc2_b")
 LAYER_I8 = ("attn", "proj", "fc", "fc2")
 

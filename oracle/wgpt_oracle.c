@@ -343,6 +343,57 @@ void ref_dequantize_js(int count, const int32_t* packed, float absmax, float* w)
 }
 
 /* ---------------------------------------------------------------------------
+ * Token selection, model.js:81-85.
+ * selectTopK (globals.js:66-74): the (value, index) pairs are sorted with the comparator
+ * b.value - a.value; Array.prototype.sort is stable, so equal values keep ascending index.
+ * Here: bottom-up merge sort taking from the left run on ties (stable).
+ * cpuSoftmax (globals.js:59-64): max over the k values; exp((x - max) / temperature) in
+ * float64; sum by reduce from 0, left to right; each term divided by the sum.
+ * sampleFromDistribution (globals.js:47-57): running sum, first i with u < sum, else k-1.
+ * ------------------------------------------------------------------------- */
+int ref_sample_topk(int V, int top_k, double temperature, double u, const float* logits, int32_t* ids, double* probs) {
+  int32_t* a = (int32_t*)malloc(sizeof(int32_t) * (size_t)V);
+  int32_t* b = (int32_t*)malloc(sizeof(int32_t) * (size_t)V);
+  for (int i = 0; i < V; ++i) a[i] = i;
+  for (int width = 1; width < V; width *= 2) {
+    for (int lo = 0; lo < V; lo += 2 * width) {
+      int mid = lo + width < V ? lo + width : V;
+      int hi = lo + 2 * width < V ? lo + 2 * width : V;
+      int i = lo, j = mid, o = lo;
+      while (i < mid && j < hi) {
+        /* comparator(left, right) = right.value - left.value > 0 moves right first */
+        if (logits[a[j]] > logits[a[i]]) b[o++] = a[j++];
+        else b[o++] = a[i++];
+      }
+      while (i < mid) b[o++] = a[i++];
+      while (j < hi) b[o++] = a[j++];
+    }
+    int32_t* t = a; a = b; b = t;
+  }
+  const int k = top_k < V ? top_k : V;
+  double* e = (double*)malloc(sizeof(double) * (size_t)k);
+  double mx = -INFINITY;
+  for (int i = 0; i < k; ++i) if ((double)logits[a[i]] > mx) mx = (double)logits[a[i]];
+  double sum = 0.0;
+  for (int i = 0; i < k; ++i) {
+    e[i] = exp(((double)logits[a[i]] - mx) / temperature);
+    sum = sum + e[i];
+  }
+  double cum = 0.0;
+  int pick = k - 1, found = 0;
+  for (int i = 0; i < k; ++i) {
+    const double p = e[i] / sum;
+    if (probs) probs[i] = p;
+    if (ids) ids[i] = a[i];
+    cum += p;
+    if (!found && u < cum) { pick = i; found = 1; }
+  }
+  const int chosen = a[pick];
+  free(a); free(b); free(e);
+  return chosen;
+}
+
+/* ---------------------------------------------------------------------------
  * GPT.run(), model.js:118-240.
  *   r = embed
  *   per layer: a = attention(LN1(r)); r = a + r; m = fc2(gelu(fc(LN2(r)))); r = m + r

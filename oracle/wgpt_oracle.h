@@ -73,6 +73,12 @@ float ref_quantize_global(int count, const float* w, int32_t* packed);
 /* dequantizeMatrix other/int8-gemm.js:48-62 (double arithmetic, one rounding) */
 void ref_dequantize_js(int count, const int32_t* packed, float absmax, float* w);
 
+/* Token selection of GPT.generate, model.js:81-85: selectTopK (globals.js:66-74, stable
+ * sort by descending value), cpuSoftmax (globals.js:59-64, float64, temperature inside the
+ * exponent), sampleFromDistribution (globals.js:47-57) with `u` for Math.random().
+ * ids[k], probs[k] (k = min(top_k, V)) may be NULL. Returns the chosen index. */
+int ref_sample_topk(int V, int top_k, double temperature, double u, const float* logits, int32_t* ids, double* probs);
+
 /* Whole model, GPT.run() model.js:104-241. Weight layout is the reference's
  * on-disk one: linear weights [in,out] row-major, c_attn fused [d,3d]. */
 typedef struct {

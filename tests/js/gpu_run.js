@@ -33,6 +33,15 @@ async function main() {
   let first = 0;
   for (let i = 1; i < lg.length; i++) if (lg[i] > lg[first]) first = i;
   out.greedy = [first].concat(Array.from(gpt.decodeGreedy(first, 9)));
+  // token selection on the device: one buffer-level call, then a sampled continuation
+  const probe = new Float32Array([0.5, 2.0, -1.0, 2.0, 1.5]);
+  const pb = w.initTensor(probe, [5]);
+  const sel = w.native.sampleTopK(5, 3, 0.5, 0.6, pb.handle);
+  out.select = { id: sel.id, topKIndices: Array.from(sel.topKIndices), probs: Array.from(sel.probs) };
+  pb.destroy();
+  await gpt.run(tokens.slice(0, 8));
+  out.draws = [0.05, 0.5, 0.95, 0.3];
+  out.sampled = Array.from(gpt.decodeSample(first, 4, 0.9, out.draws));
   gpt.unloadBuffers();
   w.destroyOperations();
   console.log(JSON.stringify(out));

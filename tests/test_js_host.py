@@ -78,3 +78,14 @@ def test_js_gpt_on_gpu_matches_oracle():
         nxt = int(np.argmax(ref.forward(p, w, np.array(hist, np.int32))))
         assert nxt == out["generated"][i]
         hist.append(nxt)
+    # token selection on the device, through the addon (globals.js:47-74)
+    want_id, want_ids, want_p = ref.sample_topk(np.array([0.5, 2.0, -1.0, 2.0, 1.5], np.float32), 3, 0.5, 0.6)
+    assert out["select"]["id"] == want_id and out["select"]["topKIndices"] == [int(i) for i in want_ids]
+    assert np.allclose(out["select"]["probs"], want_p, rtol=1e-12)
+    hist = [int(t) for t in tokens[:8]] + [out["greedy"][0]]
+    for i, u in enumerate(out["draws"]):
+        lg = ref.forward(p, w, np.array(hist, np.int32))
+        want, ids, pr = ref.sample_topk(lg, 4, 0.9, u)
+        assert out["sampled"][i] == want or np.min(np.abs(np.cumsum(pr) - u)) < 1e-3
+        hist.append(out["sampled"][i])
+

@@ -55,12 +55,14 @@ _SIGNATURES = {
     "wgpt_embed": ([_ip, _int, _int, _int, _u64, _u64, _u64], True),
     "wgpt_deembed": ([_int, _int, _int, _u64, _u64, _u64], True),
     "wgpt_attention": ([_int, _int, C.c_float, _int, _int] + [_u64] * 10, True),
+    "wgpt_sample_topk": ([_int, _int, C.c_double, C.c_double, _u64, _ip, _ip, C.POINTER(C.c_double)], True),
     "wgpt_model_create": ([C.POINTER(Params), C.POINTER(_u64)], True),
     "wgpt_model_set_tensor": ([_u64, C.c_char_p, _vp, _sz], True),
     "wgpt_model_finalize": ([_u64], True),
     "wgpt_prefill": ([_u64, _ip, _int, _fp], True),
     "wgpt_decode": ([_u64, C.c_int32, _fp], True),
     "wgpt_decode_greedy": ([_u64, C.c_int32, _int, _ip, _fp], True),
+    "wgpt_decode_sample": ([_u64, C.c_int32, _int, _int, C.c_double, C.POINTER(C.c_double), _ip, _fp], True),
     "wgpt_model_reset_cache": ([_u64], True),
     "wgpt_model_position": ([_u64, C.POINTER(_int)], True),
     "wgpt_model_tap": ([_u64, C.c_char_p, _fp, _sz], True),

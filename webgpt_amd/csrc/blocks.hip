@@ -15,7 +15,7 @@ struct Scratch {
   void* ptr = nullptr;
   size_t bytes = 0;
 };
-static Scratch g_scratch[4];
+static Scratch g_scratch[5];
 
 static int scratch(int slot, size_t bytes, void** out) {
   Scratch& s = g_scratch[slot];
@@ -182,6 +182,35 @@ int wgpt_softmax(int M, int N, wgpt_buf x, wgpt_buf out) {
   if (px == po) return fail(WGPT_ERR_ARG, "wgpt_softmax: out must not alias x");
   hipError_t e = launch_softmax(M, N, px, po, rt().stream);
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "softmax launch: %s", hipGetErrorString(e));
+  return WGPT_OK;
+}
+
+int wgpt_sample_topk(int V, int top_k, double temperature, double u, wgpt_buf logits, int32_t* id, int32_t* ids,
+                     double* probs) {
+  WGPT_REQUIRE_INIT();
+  if (V < 1 || V > SAMPLE_MAX_V) return fail(WGPT_ERR_ARG, "wgpt_sample_topk: V must be in [1, %d]", SAMPLE_MAX_V);
+  if (top_k < 1 || top_k > SAMPLE_MAX_K) return fail(WGPT_ERR_ARG, "wgpt_sample_topk: top_k must be in [1, %d]", SAMPLE_MAX_K);
+  if (!(temperature > 0.0)) return fail(WGPT_ERR_ARG, "wgpt_sample_topk: temperature must be positive");
+  if (!(u >= 0.0 && u < 1.0)) return fail(WGPT_ERR_ARG, "wgpt_sample_topk: u must be in [0, 1)");
+  if (!id) return fail(WGPT_ERR_ARG, "wgpt_sample_topk: id is NULL");
+  const float* pl = F(logits, (size_t)V, "wgpt_sample_topk(logits)");
+  if (!pl) return WGPT_ERR_ARG;
+  const int k = top_k < V ? top_k : V;
+  // scratch: [u | probs[k]] doubles, then [tok | ids[k]] ints
+  void* ws;
+  int rc = scratch(4, sizeof(double) * (size_t)(1 + k) + sizeof(int32_t) * (size_t)(1 + k), &ws);
+  if (rc) return rc;
+  double* du = (double*)ws;
+  double* dprobs = du + 1;
+  int32_t* dtok = (int32_t*)(dprobs + k);
+  int32_t* dids = dtok + 1;
+  WGPT_HIP(hipMemcpyAsync(du, &u, sizeof(double), hipMemcpyHostToDevice, rt().stream));
+  hipError_t e = launch_sample_topk(V, k, temperature, du, pl, dtok, nullptr, 0, dids, dprobs, rt().stream);
+  if (e != hipSuccess) return fail(WGPT_ERR_HIP, "sample_topk launch: %s", hipGetErrorString(e));
+  WGPT_HIP(hipMemcpyAsync(id, dtok, sizeof(int32_t), hipMemcpyDeviceToHost, rt().stream));
+  if (ids) WGPT_HIP(hipMemcpyAsync(ids, dids, sizeof(int32_t) * (size_t)k, hipMemcpyDeviceToHost, rt().stream));
+  if (probs) WGPT_HIP(hipMemcpyAsync(probs, dprobs, sizeof(double) * (size_t)k, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
   return WGPT_OK;
 }
 

@@ -53,6 +53,13 @@ hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const 
 hipError_t launch_kv_append(int T, int d, int hs, int ctx, int pos0, const float* qkv, float* Kc, float* Vc, hipStream_t s);
 // Copies rows of src (row stride lds, `cols` floats wide) to dst (row stride ldd).
 hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float* dst, int ldd, hipStream_t s);
+// Top-k / temperature / inverse-CDF selection of one token on the device (globals.js:47-74,
+// model.js:81-85); *u is the uniform draw, device memory. tok[0] and out[slot] (optional) get
+// the id, ids[k] / probs[k] (optional) the selected indices and their probabilities.
+constexpr int SAMPLE_MAX_V = 262144;
+constexpr int SAMPLE_MAX_K = 1024;
+hipError_t launch_sample_topk(int V, int k, double temperature, const double* u, const float* logits, int32_t* tok,
+                              int32_t* out, int slot, int32_t* ids, double* probs, hipStream_t s);
 // tok[0] = argmax(logits[0..V)) with the lowest index on ties; also stored to out[slot].
 hipError_t launch_argmax(int V, const float* logits, int32_t* tok, int32_t* out, int slot, hipStream_t s);
 

@@ -674,6 +674,110 @@ __global__ __launch_bounds__(WG) void kv_append_kernel(int d, int hs, int ctx, i
   }
 }
 
+// Token selection of GPT.generate (model.js:81-85) on the device, one workgroup:
+//   selectTopK (globals.js:66-74): stable descending sort of (value, index), first k;
+//     here k rounds of arg-max with the lowest index among equal values;
+//   cpuSoftmax (globals.js:59-64) of those k logits in float64:
+//     exp((x - max) / temperature), summed left to right, divided by the sum;
+//   sampleFromDistribution (globals.js:47-57): first i with u < p_0 + .. + p_i, else k - 1;
+//     u is the caller's uniform draw in [0, 1) (the reference's Math.random()).
+// The chosen id goes to tok[0] (input of the next decode step) and out[slot]; ids/probs
+// (optional) receive the k selected indices and their probabilities.
+__device__ __forceinline__ bool better(float ov, int oi, float cv, int ci) {
+  return oi != 0x7fffffff && (ci == 0x7fffffff || ov > cv || (ov == cv && oi < ci));
+}
+
+__global__ __launch_bounds__(1024) void sample_topk_kernel(int V, int k, double temperature, const double* __restrict__ u,
+                                                            const float* __restrict__ logits, int32_t* tok, int32_t* out, int slot,
+                                                            int32_t* ids, double* probs) {
+  __shared__ unsigned taken[SAMPLE_MAX_V / 32];
+  __shared__ float wv[16];
+  __shared__ int wi[16];
+  __shared__ float sel_v[SAMPLE_MAX_K];
+  __shared__ int sel_i[SAMPLE_MAX_K];
+  __shared__ double ev[SAMPLE_MAX_K];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < (V + 31) / 32; i += 1024) taken[i] = 0u;
+  if (k > V) k = V;
+  // this thread's candidate: the best not yet taken element of its stride
+  auto scan = [&](float& best, int& besti) {
+    best = -INFINITY;
+    besti = 0x7fffffff;
+    for (int i = tid; i < V; i += 1024) {
+      if (taken[i >> 5] & (1u << (i & 31))) continue;
+      const float v = logits[i];
+      if (v > best || besti == 0x7fffffff) {
+        best = v;
+        besti = i;
+      }
+    }
+  };
+  __syncthreads();
+  float best;
+  int besti;
+  scan(best, besti);
+  for (int r = 0; r < k; ++r) {
+    float cv = best;
+    int ci = besti;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(cv, off);
+      const int oi = __shfl_xor(ci, off);
+      if (better(ov, oi, cv, ci)) {
+        cv = ov;
+        ci = oi;
+      }
+    }
+    if (lane == 0) {
+      wv[wave] = cv;
+      wi[wave] = ci;
+    }
+    __syncthreads();
+    cv = wv[0];
+    ci = wi[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w)
+      if (better(wv[w], wi[w], cv, ci)) {
+        cv = wv[w];
+        ci = wi[w];
+      }
+    // every thread knows the winner; its owner marks it and looks for its next candidate
+    if (tid == 0) {
+      sel_v[r] = cv;
+      sel_i[r] = ci;
+    }
+    if ((ci & 1023) == tid) {
+      taken[ci >> 5] |= 1u << (ci & 31);
+      scan(best, besti);
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const double mx = (double)sel_v[0];
+    double sum = 0.0;
+    for (int i = 0; i < k; ++i) {
+      ev[i] = exp(((double)sel_v[i] - mx) / temperature);
+      sum += ev[i];
+    }
+    const double rnd = *u;
+    double cum = 0.0;
+    int pick = k - 1;
+    bool found = false;
+    for (int i = 0; i < k; ++i) {
+      const double p = ev[i] / sum;
+      if (probs) probs[i] = p;
+      if (ids) ids[i] = sel_i[i];
+      cum += p;
+      if (!found && rnd < cum) {
+        pick = i;
+        found = true;
+      }
+    }
+    tok[0] = sel_i[pick];
+    if (out) out[slot] = sel_i[pick];
+  }
+}
+
 // Greedy selection: selectTopK with top_k = 1 (globals.js:66-74) is a stable
 // descending sort, i.e. the largest logit with the lowest index on ties.
 __global__ __launch_bounds__(1024) void argmax_kernel(int V, const float* __restrict__ logits, int32_t* tok, int32_t* out,
@@ -848,6 +952,13 @@ hipError_t launch_copy_rows(int rows, int cols, const float* src, int lds, float
 
 hipError_t launch_kv_append(int T, int d, int hs, int ctx, int pos0, const float* qkv, float* Kc, float* Vc, hipStream_t s) {
   kv_append_kernel<<<T, WG, 0, s>>>(d, hs, ctx, pos0, qkv, Kc, Vc);
+  return hipGetLastError();
+}
+
+hipError_t launch_sample_topk(int V, int k, double temperature, const double* u, const float* logits, int32_t* tok,
+                              int32_t* out, int slot, int32_t* ids, double* probs, hipStream_t s) {
+  if (V < 1 || V > SAMPLE_MAX_V || k < 1 || k > SAMPLE_MAX_K) return hipErrorInvalidValue;
+  sample_topk_kernel<<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
   return hipGetLastError();
 }
 

@@ -45,6 +45,8 @@ struct Model {
   float* taps = nullptr;         // [(2+6L)][maxT][d]
   int32_t* tok_dev = nullptr;    // [maxT] token ids of the current call
   int32_t* out_tok_dev = nullptr;  // [ctx] ids chosen by the greedy loop
+  int32_t* out_samp_dev = nullptr; // [ctx] ids chosen by the sampling loop
+  double* u_dev = nullptr;         // [ctx] uniform draws of the sampling loop
 
   // persistent whole-token decode (decode_mode 1): slab-layout weights, exchange buffers
   bool persist_ok = false;

@@ -426,6 +426,8 @@ int wgpt_model_finalize(wgpt_model h) {
   if ((rc = dev_alloc(m, (size_t)m->V * f, (void**)&m->logits))) return rc;
   if ((rc = dev_alloc(m, T * sizeof(int32_t), (void**)&m->tok_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
+  if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_samp_dev))) return rc;
+  if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(double), (void**)&m->u_dev))) return rc;
   size_t ws = gemv_workspace_floats(GEMV_MAX_ROWS, 4 * (int)d, (int)d);
   const size_t ws2 = gemv_workspace_floats(GEMV_MAX_ROWS, (int)d, 4 * (int)d);
   if (ws2 > ws) ws = ws2;
@@ -520,6 +522,46 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
     if (rc) return rc;
   }
   m->pos += steps;
+  return WGPT_OK;
+}
+
+int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double temperature, const double* u,
+                       int32_t* out_tokens, float* logits) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_sample: model not finalised");
+  if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: token id %d outside [0, %d)", token, m->V);
+  if (steps < 1 || !out_tokens || !u) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: steps >= 1, u and out_tokens required");
+  if (top_k < 1 || top_k > SAMPLE_MAX_K) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: top_k must be in [1, %d]", SAMPLE_MAX_K);
+  if (m->V > SAMPLE_MAX_V) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: vocabulary above %d", SAMPLE_MAX_V);
+  if (!(temperature > 0.0)) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: temperature must be positive");
+  for (int i = 0; i < steps; ++i)
+    if (!(u[i] >= 0.0 && u[i] < 1.0)) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: u[%d] must be in [0, 1)", i);
+  if (m->pos + steps > m->ctx)
+    return fail(WGPT_ERR_STATE, "wgpt_decode_sample: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipMemcpyAsync(m->u_dev, u, sizeof(double) * (size_t)steps, hipMemcpyHostToDevice, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
+  const bool persistent = m->decode_mode == 1;
+  const int k = top_k < m->V ? top_k : m->V;
+  for (int i = 0; i < steps; ++i) {
+    // one token per launch: the sampled id in tok_dev[0] is the next launch's input
+    int rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+    if (rc) return rc;
+    LAUNCH(launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream));
+    m->pos += 1;
+  }
+  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
+  WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
+  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  if (persistent) {
+    int rc = check_persistent(m);
+    if (rc) return rc;
+  }
   return WGPT_OK;
 }
 

@@ -29,7 +29,8 @@ void* g_lib = nullptr;
   X(wgpt_model_set_tensor) X(wgpt_model_finalize) X(wgpt_prefill) X(wgpt_decode) X(wgpt_decode_greedy)  \
   X(wgpt_model_reset_cache) X(wgpt_model_position) X(wgpt_model_tap) X(wgpt_model_last_gpu_ms)          \
   X(wgpt_model_decode_bytes) X(wgpt_model_set_decode_mode) X(wgpt_model_destroy) X(wgpt_synth_normal)   \
-  X(wgpt_synth_tokens) X(wgpt_synth_int8_packed) X(wgpt_synth_uniform) X(wgpt_synth_tensor_id)
+  X(wgpt_synth_tokens) X(wgpt_synth_int8_packed) X(wgpt_synth_uniform) X(wgpt_synth_tensor_id)   \
+  X(wgpt_decode_sample) X(wgpt_sample_topk)
 
 #define DECL(name) decltype(&::name) p_##name = nullptr;
 WGPT_FUNCS(DECL)
@@ -278,6 +279,47 @@ FN(DecodeGreedy) {  // (model, token, steps) -> Int32Array ids
   if (failed(env, p_wgpt_decode_greedy(m, tok, steps, (int32_t*)p, nullptr))) return nullptr;
   return ta;
 }
+FN(DecodeSample) {  // (model, token, topK, temperature, Float64Array u) -> Int32Array ids, one per draw
+  Args a(env, info);
+  uint64_t m = a.u64(0);
+  int tok = a.i32(1), top_k = a.i32(2);
+  double temperature = a.num(3);
+  if (!a.ok) return nullptr;
+  napi_typedarray_type type;
+  size_t steps = 0;
+  void* udata = nullptr;
+  if (a.argc < 5 || napi_get_typedarray_info(env, a.argv[4], &type, &steps, &udata, nullptr, nullptr) != napi_ok || type != napi_float64_array || steps < 1)
+    return throw_error(env, "wgpt_decode_sample: u must be a non-empty Float64Array");
+  napi_value ab, ta;
+  void* p;
+  if (napi_create_arraybuffer(env, sizeof(int32_t) * steps, &p, &ab) != napi_ok) return throw_error(env, "webgpt_amd: out of memory");
+  napi_create_typedarray(env, napi_int32_array, steps, ab, 0, &ta);
+  if (failed(env, p_wgpt_decode_sample(m, tok, (int)steps, top_k, temperature, (const double*)udata, (int32_t*)p, nullptr))) return nullptr;
+  return ta;
+}
+FN(SampleTopK) {  // (V, topK, temperature, u, logitsBuffer) -> {id, topKIndices: Int32Array, probs: Float64Array}
+  Args a(env, info);
+  int V = a.i32(0), top_k = a.i32(1);
+  double temperature = a.num(2), u = a.num(3);
+  uint64_t buf = a.u64(4);
+  if (!a.ok) return nullptr;
+  if (top_k < 1 || V < 1) return throw_error(env, "wgpt_sample_topk: V and top_k must be positive");
+  const size_t k = (size_t)(top_k < V ? top_k : V);
+  napi_value ab_i, ta_i, ab_p, ta_p, obj, idv;
+  void *pi, *pp;
+  if (napi_create_arraybuffer(env, sizeof(int32_t) * k, &pi, &ab_i) != napi_ok || napi_create_arraybuffer(env, sizeof(double) * k, &pp, &ab_p) != napi_ok)
+    return throw_error(env, "webgpt_amd: out of memory");
+  napi_create_typedarray(env, napi_int32_array, k, ab_i, 0, &ta_i);
+  napi_create_typedarray(env, napi_float64_array, k, ab_p, 0, &ta_p);
+  int32_t id = 0;
+  if (failed(env, p_wgpt_sample_topk(V, top_k, temperature, u, buf, &id, (int32_t*)pi, (double*)pp))) return nullptr;
+  napi_create_object(env, &obj);
+  napi_create_int32(env, id, &idv);
+  napi_set_named_property(env, obj, "id", idv);
+  napi_set_named_property(env, obj, "topKIndices", ta_i);
+  napi_set_named_property(env, obj, "probs", ta_p);
+  return obj;
+}
 FN(ModelTap) {  // (model, name, nFloats) -> Float32Array
   Args a(env, info);
   uint64_t m = a.u64(0);
@@ -353,7 +395,7 @@ napi_value InitModule(napi_env env, napi_value exports) {
       {"modelCreate", ModelCreate}, {"modelSetTensor", ModelSetTensor}, {"modelFinalize", ModelFinalize},
       {"modelDestroy", ModelDestroy}, {"modelResetCache", ModelResetCache}, {"modelSetDecodeMode", ModelSetDecodeMode},
       {"modelPosition", ModelPosition}, {"modelLastGpuMs", ModelLastGpuMs}, {"modelDecodeBytes", ModelDecodeBytes},
-      {"prefill", Prefill}, {"decode", Decode}, {"decodeGreedy", DecodeGreedy}, {"modelTap", ModelTap},
+      {"prefill", Prefill}, {"decode", Decode}, {"decodeGreedy", DecodeGreedy}, {"decodeSample", DecodeSample}, {"sampleTopK", SampleTopK}, {"modelTap", ModelTap},
       {"synthNormal", SynthNormal}};
   for (const auto& e : table) {
     napi_value fn;

@@ -104,6 +104,17 @@ class GPT {
     return ids;
   }
 
+  // Sampled continuation on the device: one token per entry of `draws` (uniform numbers in
+  // [0, 1), what the reference takes from Math.random()), chosen as generate() chooses
+  // (model.js:81-85) without reading the logits back.
+  decodeSample(token, topK, temperature, draws) {
+    const u = Float64Array.from(draws);
+    const ids = native.decodeSample(this.model.handle, token, topK, temperature, u);
+    this._history = this._history.concat([token], Array.from(ids.slice(0, u.length - 1)));
+    this.lastGpuMs = native.modelLastGpuMs(this.model.handle);
+    return ids;
+  }
+
   // The reference's pass list (model.js:118-240) built block by block from separately
   // uploaded weights and replayed through the per-block entry points.
   async runBlocks(idx, weights) {

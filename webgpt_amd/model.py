@@ -210,6 +210,19 @@ class GPT:
         self._update_ms()
         return (out, logits) if want_logits else out
 
+    def decode_sample(self, token, steps, top_k, temperature, u):
+        """`steps` tokens chosen on the device as GPT.generate chooses them (model.js:81-85),
+        u[i] standing for the i-th Math.random() draw; the logits never leave the device."""
+        u = np.ascontiguousarray(u, np.float64)
+        if u.shape != (steps,):
+            raise ValueError("decode_sample: one uniform draw per step")
+        out = np.empty(steps, np.int32)
+        _lib.call("wgpt_decode_sample", self._handle, int(token), steps, int(top_k), float(temperature),
+                  u.ctypes.data_as(C.POINTER(C.c_double)), out.ctypes.data_as(_IP), None)
+        self._history += [int(token)] + [int(t) for t in out[:-1]]
+        self._update_ms()
+        return out
+
     def _update_ms(self):
         ms = C.c_float(0)
         _lib.call("wgpt_model_last_gpu_ms", self._handle, C.byref(ms))
