@@ -14,6 +14,7 @@ const { performance } = require("perf_hooks");
 const native = require("./native.js");
 const { Device, initTensor, runPasses } = require("./instructions.js");
 const G = require("./globals.js");
+const { GPT2Tokenizer, SimpleTokenizer } = require("./tokenizer.js");
 
 class GPT {
   constructor(folder, type, options = {}) {
@@ -34,6 +35,7 @@ class GPT {
     this._tensors = options.tensors;  // Map or object name -> TypedArray, instead of files
     this._paramsIn = options.params;
     this._flags = options.flags || 0;
+    this._tokenization = options.tokenization;
     this._history = [];
     this.lastGpuMs = 0;
   }
@@ -43,6 +45,18 @@ class GPT {
     this.device = new Device(0);
     G.initializeOperations(this.device);
     [this.model, this.params] = await this.loadModel(this.folder);
+    // model.js:33-34: the tokenizer of the model type, from options.tokenization (the folder
+    // the reference calls weights/tokenization) unless one was handed in
+    if (!this.tokenizer && this._tokenization) {
+      const dir = this._tokenization;
+      if (this.tokenizerType == "bpe") {
+        const tokens = path.join(dir, "gpt_tokens.json");
+        const real = fs.existsSync(tokens) && fs.readFileSync(tokens, "utf8").trimStart().startsWith("{");
+        this.tokenizer = await new GPT2Tokenizer().load(path.join(dir, "vocab.bpe"), real ? tokens : undefined);
+      } else {
+        this.tokenizer = await new SimpleTokenizer().load(path.join(dir, "simple_tokens.json"));
+      }
+    }
     if (this.tokenizerType == "bpe") {
       this.defaultPrompt = `What is the answer to life, the universe, and everything?\n`;
       this.defaultTopK = 3;

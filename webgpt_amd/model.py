@@ -68,7 +68,7 @@ def read_tensor(weightsFolder, name, params):
 
 
 class GPT:
-    def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0):
+    def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0, tokenization=None):
         self.folder = folder
         self.tokenizerType = type
         self.initialized = False
@@ -86,6 +86,7 @@ class GPT:
         self._params_in = params
         self._flags = flags
         self._device_index = device_index
+        self._tokenization = tokenization
         self._handle = None
         self._history = []
         self.lastGpuMs = 0.0
@@ -99,6 +100,17 @@ class GPT:
         self.device = blocks.Device(self._device_index)  # raises if no gfx950 device: "WebGPU is not supported"
         blocks.initializeOperations(self.device)
         self.model, self.params = self.loadModel(self.folder)
+        # model.js:33-34: the tokenizer of the model type, from `tokenization` (the folder the
+        # reference calls weights/tokenization) unless one was handed in
+        if self.tokenizer is None and self._tokenization is not None:
+            from . import tokenizer as tk
+            d = self._tokenization
+            if self.tokenizerType == "bpe":
+                tokens = os.path.join(d, "gpt_tokens.json")
+                real = os.path.exists(tokens) and open(tokens, encoding="utf-8").read(64).lstrip().startswith("{")
+                self.tokenizer = tk.GPT2Tokenizer().load(os.path.join(d, "vocab.bpe"), tokens if real else None)
+            else:
+                self.tokenizer = tk.SimpleTokenizer().load(os.path.join(d, "simple_tokens.json"))
         if self.tokenizerType == "bpe":
             self.defaultPrompt = "What is the answer to life, the universe, and everything?\n"
             self.defaultTopK, self.defaultTemperature, self.defaultTokens = 3, 1, 30
