@@ -669,34 +669,47 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
             m = fmaxf(m, sc[i]);
           }
         }
-        if (sub == 0) sh.red[g16] = m;
-        __syncthreads();
-#pragma unroll
-        for (int v = 0; v < 32; ++v) m = fmaxf(m, sh.red[v]);
+        // softmax numerators against the maximum of this group of 16 lanes (its keys only)
         float l = 0.f;
         float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m > -INFINITY) {
 #pragma unroll
-          for (int i = 0; i < MAXKV; ++i) {
-            if (i < nkv) {
-              const float p = sc[i] > -INFINITY ? fast_exp(sc[i] - m) : 0.f;
-              l += p;
-              o.x += p * vreg[i].x; o.y += p * vreg[i].y; o.z += p * vreg[i].z; o.w += p * vreg[i].w;
-            }
+        for (int i = 0; i < MAXKV; ++i) {
+          if (i < nkv) {
+            const float p = sc[i] > -INFINITY ? fast_exp(sc[i] - m) : 0.f;
+            l += p;
+            o.x += p * vreg[i].x; o.y += p * vreg[i].y; o.z += p * vreg[i].z; o.w += p * vreg[i].w;
           }
         }
-        // the 32 key groups combine through LDS
-        *reinterpret_cast<float4*>(part + g16 * (HS + 4) + sub * 4) = o;
-        if (sub == 0) part[g16 * (HS + 4) + HS] = l;
+        // the four groups of a wave combine in registers (rescaled to the wave's maximum) ...
+        float mw = fmaxf(m, __shfl_xor(m, 16));
+        mw = fmaxf(mw, __shfl_xor(mw, 32));
+        const float f = m > -INFINITY ? fast_exp(m - mw) : 0.f;
+        l *= f;
+        o.x *= f; o.y *= f; o.z *= f; o.w *= f;
+        l += __shfl_xor(l, 16); o.x += __shfl_xor(o.x, 16); o.y += __shfl_xor(o.y, 16); o.z += __shfl_xor(o.z, 16); o.w += __shfl_xor(o.w, 16);
+        l += __shfl_xor(l, 32); o.x += __shfl_xor(o.x, 32); o.y += __shfl_xor(o.y, 32); o.z += __shfl_xor(o.z, 32); o.w += __shfl_xor(o.w, 32);
+        // ... and the eight waves through LDS: (o[HS], m, l) per wave
+        if (lane < 16) {
+          *reinterpret_cast<float4*>(part + wave * (HS + 4) + sub * 4) = o;
+          if (sub == 0) {
+            part[wave * (HS + 4) + HS] = mw;
+            part[wave * (HS + 4) + HS + 1] = l;
+          }
+        }
         __syncthreads();
         if (tid < HS + 2) {
-          float v = 0.f;
-          if (tid == HS) {
-            v = m;
-          } else {
-            const int c = tid < HS ? tid : HS;
-#pragma unroll 8
-            for (int g2 = 0; g2 < 32; ++g2) v += part[g2 * (HS + 4) + c];
+          float M = -INFINITY;
+#pragma unroll
+          for (int w2 = 0; w2 < NW; ++w2) M = fmaxf(M, part[w2 * (HS + 4) + HS]);
+          float v = M;
+          if (tid != HS) {
+            const int c = tid < HS ? tid : HS + 1;
+            v = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) {
+              const float mv = part[w2 * (HS + 4) + HS];
+              v += part[w2 * (HS + 4) + c] * (mv > -INFINITY ? fast_exp(mv - M) : 0.f);
+            }
           }
           publish(a.bufATT + (size_t)wg * (HS + 2) + tid, v, ep);
         }

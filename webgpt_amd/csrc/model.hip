@@ -266,7 +266,7 @@ static int setup_persistent(Model* m) {
     // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
     // curves are flat within a few percent around them and over context length);
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
-    static const int tuned[4][7] = {{16, 4, 28, 96, 24, 20, 40},    // d <= 768
+    static const int tuned[4][7] = {{16, 0, 28, 96, 24, 20, 40},    // d <= 768
                                     {20, 0, 48, 96, 28, 32, 64},    // d = 1024
                                     {20, 0, 48, 96, 4, 20, 40},     // d = 1280
                                     {40, 0, 48, 96, 32, 40, 40}};   // d = 1600, int8
