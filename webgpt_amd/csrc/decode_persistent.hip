@@ -376,8 +376,10 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
 template <class P, bool LNORM, bool AFFINE, class WS>
 __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const float* lnp, int ncols, int wave, int lane) {
   static_assert(P::WHOLE, "phase is not laid out by whole columns");
-  float4 xr[P::S];
-  input_row<P::K, LNORM, AFFINE>(xr, xs, lnp, lane);
+  // a normalised row is held in registers; a plain one is read from LDS item by item
+  float4 xr[LNORM ? P::S : 1];
+  if (LNORM) input_row<P::K, LNORM, AFFINE>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, lane);
+  const float* xl = xs + opaque(lane) * 4;
   float val = 0.f;
 #pragma unroll
   for (int cc = 0; cc < P::CW; ++cc) {
@@ -385,8 +387,9 @@ __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const
       float acc = 0.f;
 #pragma unroll
       for (int seg = 0; seg < P::S; ++seg) {
+        const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
         const float4 w = to_float4(ws.w[cc * P::S + seg]);
-        acc += (w.x * xr[seg].x + w.y * xr[seg].y) + (w.z * xr[seg].z + w.w * xr[seg].w);
+        acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
       }
       const float r = wave_sum(acc);
       val = lane == cc ? r : val;
@@ -426,6 +429,19 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
       }
     }
   });
+}
+
+// Second MLP matrix: either layout. Whole columns leave residual + column in pubE;
+// split columns leave per-wave partials in part (finished after the barrier).
+template <class P, bool I8, class WS>
+__device__ __forceinline__ void phase_e(const WS& ws, const float* xs, float* part, const float* pubC, float* pubE, int ncols,
+                                        bool fin, int fc, int wave, int lane) {
+  if constexpr (P::WHOLE) {
+    const float dot = gemv_whole<P, false, false>(ws, xs, nullptr, ncols, wave, lane);
+    if (fin) pubE[fc] = pubC[fc] + ((I8 ? dot * ws.cscale : dot) + ws.bias);
+  } else {
+    gemv_split<P>(ws, xs, part, ncols, wave, lane);
+  }
 }
 
 // Sum of the per-wave partials of local column c, in ascending wave order.
@@ -469,7 +485,7 @@ struct Phases {
   typedef Phase<3 * C::D, C::D, true> A;    // c_attn
   typedef Phase<C::D, C::D, true> Cc;       // attention c_proj
   typedef Phase<C::HID, C::D, true> Dd;     // c_fc
-  typedef Phase<C::D, C::HID, false> E;     // mlp c_proj
+  typedef Phase<C::D, C::HID, C::I8> E;      // mlp c_proj: whole columns only where an item is one register (int8)
   static constexpr int MAXI = cmax(cmax(A::IPW, Dd::IPW), cmax(Cc::IPW, E::IPW));
   // Two register sets (c_attn and c_fc in one, the two projections in the other) let a
   // phase's weights be requested a whole phase ahead, right after the poll of the
@@ -509,6 +525,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float* pubA = qkv_s + 3 * HS;   // [PA::CPW] finished c_attn columns
   float* pubC = pubA + PA::CPW;   // [PC::CPW] residual stream after the attention projection
   float* pubD = pubC + PC::CPW;   // [PD::CPW] finished c_fc columns
+  float* pubE = pubD + PD::CPW;   // [PE::CPW] residual stream after the MLP (whole-column layout only)
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
@@ -525,6 +542,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // local column this lane finishes (lane cc of wave v: column v + cc * NW)
   const int fc = wave + lane * NW;
   const bool finA = lane < PA::CW && fc < ncA, finC = lane < PC::CW && fc < ncC, finD = lane < PD::CW && fc < ncD;
+  const bool finE = lane < PE::CW && fc < ncE;
 
   // attention role: head and slice of the positions; threads form 32 key groups
   // (tid >> 4) of 16 lanes (tid & 15)
@@ -817,11 +835,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         if (DUAL) request_next();
-        gemv_split<PE>(wY, xs1, part, ncE, wave, lane);
+        phase_e<PE, I8>(wY, xs1, part, pubC, pubE, ncE, finE, fc, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
-        if (tid < ncE) publish(a.bufR2 + wg * PE::CPW + tid, pubC[tid] + finish<I8>(column_sum<PE>(part, tid), wY), ep);  // model.js:205
+        if (tid < ncE) {  // model.js:205
+          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(column_sum<PE>(part, tid), wY);
+          publish(a.bufR2 + wg * PE::CPW + tid, r2, ep);
+        }
         TRACE5(4);
         if (!DUAL) request_next();
         TRACE5(5);
@@ -990,7 +1011,7 @@ size_t lds_bytes_of() {
   constexpr int XS = (C::SD + C::SH) * SEG;
   constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;
   constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
-  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + PS::Cc::CPW + PS::Dd::CPW + 16);
+  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + 16);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
   const size_t one_per_cu = 84 * 1024;
   return need > one_per_cu ? need : one_per_cu;
