@@ -9,14 +9,10 @@
 
 namespace wgpt {
 
-#ifndef WGPT_PD_THREADS
-#define WGPT_PD_THREADS 512
-#endif
-constexpr int PD_THREADS = WGPT_PD_THREADS;  // threads per workgroup (512 or 1024)
+constexpr int PD_THREADS = 512;  // threads per workgroup
 constexpr int PD_GRID = 256;     // workgroups: one per compute unit of an MI355X
 constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase
-constexpr int PD_KEYGROUPS = PD_THREADS / 16;  // groups of 16 lanes, one key each per batch
-constexpr int PD_MAXKV = 256 / PD_KEYGROUPS;   // key batches a slice can hold: n_ctx <= PD_KEYGROUPS*PD_MAXKV*PD_SPLIT
+constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
 // [w*cpw, (w+1)*cpw) of N; a column is S segments of 256 contraction elements; the

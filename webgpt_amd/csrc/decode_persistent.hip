@@ -41,7 +41,6 @@ typedef unsigned long long u64;
 constexpr int NT = PD_THREADS;       // threads per workgroup
 constexpr int NW = NT / 64;          // waves per workgroup
 constexpr int SEG = 256;             // contraction elements per item (64 lanes x float4)
-constexpr int NPMAX = 8;             // a poll round covers up to NPMAX*NT words
 constexpr unsigned SPIN_LIMIT = 1u << 18;
 
 __device__ __forceinline__ u64 ld_word(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -63,12 +62,6 @@ __device__ __forceinline__ int opaque(int v) {
   asm volatile("" : "+v"(v));
   return v;
 }
-// Same for a wave-uniform value held in a scalar register.
-__device__ __forceinline__ int opaque_s(int v) {
-  asm volatile("" : "+s"(v));
-  return v;
-}
-
 // One data-parallel-primitive step: v (+|max) the value of another lane selected by
 // CTRL, only in the rows of ROWS; lanes without a source contribute the identity.
 template <int CTRL, int ROWS>
@@ -91,15 +84,6 @@ __device__ __forceinline__ float wave_sum(float v) {
   v = dpp_add<0x118, 0xf>(v);
   v = dpp_add<0x142, 0xa>(v);
   v = dpp_add<0x143, 0xc>(v);
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-}
-__device__ __forceinline__ float wave_max(float v) {
-  v = dpp_max<0x111, 0xf>(v);
-  v = dpp_max<0x112, 0xf>(v);
-  v = dpp_max<0x114, 0xf>(v);
-  v = dpp_max<0x118, 0xf>(v);
-  v = dpp_max<0x142, 0xa>(v);
-  v = dpp_max<0x143, 0xc>(v);
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 // Sum over each row of 16 lanes, every lane of the row gets it (row rotations).
@@ -594,7 +578,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 
       // ======================= c_attn: LN1 + QKV =======================
       {
-        constexpr int PH = PH_QKV;
+        [[maybe_unused]] constexpr int PH = PH_QKV;
         if (li > 0) {
           poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0]);
           if (!FOLD) deposit_ln<D>(lnreg, lnp);
@@ -735,7 +719,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
-        constexpr int PH = PH_PROJ;
+        [[maybe_unused]] constexpr int PH = PH_PROJ;
         poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3]);
         __syncthreads();
         wait_loads();
@@ -791,7 +775,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 
       // ======================= c_fc: LN2 + fc + GELU =======================
       {
-        constexpr int PH = PH_FC;
+        [[maybe_unused]] constexpr int PH = PH_FC;
         poll_words<D>(a.bufR1, ep, xs0, a.err, a.delay[4]);
         if (!FOLD) deposit_ln<D>(lnreg, lnp);
         __syncthreads();
@@ -817,7 +801,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 
       // ======================= mlp c_proj: fc2 + residual =======================
       {
-        constexpr int PH = PH_FC2;
+        [[maybe_unused]] constexpr int PH = PH_FC2;
         // weights of the phase after this one: the next layer's c_attn share with its
         // LayerNorm; after the last layer the final LayerNorm (and, with two register
         // sets, already the first layer's share for the next token)
