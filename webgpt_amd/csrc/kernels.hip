@@ -654,6 +654,164 @@ __global__ __launch_bounds__(WG) void attention_tile_kernel(int Tq, int pos0, fl
   if (i < Tq) st4(out + (size_t)i * ldo + h * AHS + 4 * c, make_float4(o.x / l, o.y / l, o.z / l, o.w / l));
 }
 
+// ---------------------------------------------------------------------------
+// Prefill attention on the matrix cores (head size 64, at least 32 queries).
+// A workgroup owns 32 queries of one head; its four waves split the visible keys
+// into contiguous runs of 32-key tiles and are merged at the end (flash-decoding).
+// Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with
+// v_mfma_f32_32x32x2_f32: an accumulator then holds, per lane, 16 keys (or output
+// dimensions) of ONE query (column l % 32), so the softmax over keys is a reduction
+// over a lane's own registers plus one exchange with lane l ^ 32, the rescaling of
+// O by exp(m_old - m_new) is a per-lane scalar, and the probabilities are already
+// in the operand layout of the second product:
+//   accumulator register r of lane l is row (r/4)*8 + (l/32)*4 + r%4, column l%32;
+//   operand lane l supplies A[row l%32][k l/32] and B[k l/32][col l%32] per step.
+// The contraction index of either product may be visited in any order as long as
+// both operands agree: QK^T steps through dimension (l/32)*32 + i at step i (each
+// lane's 32 dimensions are contiguous in memory), PV through key
+// (i/4)*8 + (l/32)*4 + i%4 at step i (exactly the key that register i holds).
+// Scores are scaled by folding 1/sqrt(hs) into Q.
+// ---------------------------------------------------------------------------
+constexpr int AMQ = 32;        // queries per workgroup
+constexpr int AMK = 32;        // keys per tile
+constexpr int AMKST = AHS + 4; // row stride of a staged K tile (conflict-free 128-bit reads by 32 rows)
+constexpr int AM_WAVE_FLOATS = AMK * AMKST + AMK * AHS;  // K tile + V tile of one wave
+constexpr int AMOST = AMQ + 1; // row stride of a wave's O^T[dim][query] in the merge
+
+__global__ __launch_bounds__(WG) void attention_mfma_kernel(int Tq, int pos0, float scale, const float* __restrict__ q, int ldq,
+                                                             const float* __restrict__ Kc, const float* __restrict__ Vc,
+                                                             size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
+  extern __shared__ __attribute__((aligned(16))) float am_lds[];
+  const int h = blockIdx.x, q0 = blockIdx.y * AMQ;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  float* Ks = am_lds + wave * AM_WAVE_FLOATS;
+  float* Vs = Ks + AMK * AMKST;
+  const float* kbase = Kc + h * hstride;
+  const float* vbase = Vc + h * hstride;
+  const int qrow = q0 + l32;                 // this lane's query (may be >= Tq in the last block)
+  const int qpos = pos0 + qrow;              // keys 0..qpos are visible to it
+  const int qlast = q0 + AMQ - 1 < Tq - 1 ? q0 + AMQ - 1 : Tq - 1;
+  const int nkeys = pos0 + qlast + 1;        // keys any query of the block sees
+  const int nt = (nkeys + AMK - 1) / AMK;
+  const int per = (nt + NWAVE - 1) / NWAVE;
+  const int tb = wave * per;
+  const int te = tb + per < nt ? tb + per : nt;
+
+  float qf[32];  // scaled Q[qrow][hh*32 + i]
+  {
+    const float* qp = q + (size_t)(qrow < Tq ? qrow : Tq - 1) * ldq + h * AHS + hh * 32;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float4 v = ld4(qp + 4 * j);
+      qf[4 * j] = v.x * scale; qf[4 * j + 1] = v.y * scale; qf[4 * j + 2] = v.z * scale; qf[4 * j + 3] = v.w * scale;
+    }
+  }
+  float m = -INFINITY, lsum = 0.f;
+  f32x16 o0, o1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { o0[r] = 0.f; o1[r] = 0.f; }
+
+  for (int t = tb; t < te; ++t) {
+    const int k0 = t * AMK;
+    // stage the K and V tiles of this wave: 32 rows x 16 float4 each, 8 per lane; rows past the end are zero
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int f = lane + 64 * j, row = f >> 4, c4 = f & 15;
+      float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), vv = kv;
+      if (k0 + row < nkeys) {
+        kv = ld4(kbase + (size_t)(k0 + row) * ldkv + 4 * c4);
+        vv = ld4(vbase + (size_t)(k0 + row) * ldkv + 4 * c4);
+      }
+      st4(Ks + row * AMKST + 4 * c4, kv);
+      st4(Vs + row * AHS + 4 * c4, vv);
+    }
+    __builtin_amdgcn_wave_barrier();  // the tiles are private to the wave: LDS operations of a wave complete in order
+    // S^T[key][query] = sum_dim K[key][dim] Q[query][dim]
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    {
+      const float* kr = Ks + l32 * AMKST + hh * 32;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float4 kv = ld4(kr + 4 * j);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qf[4 * j], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qf[4 * j + 1], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qf[4 * j + 2], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qf[4 * j + 3], sacc, 0, 0, 0);
+      }
+    }
+    // causal mask and the running maximum of this lane's query
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + (r >> 2) * 8 + hh * 4 + (r & 3);
+      sacc[r] = key <= qpos ? sacc[r] : -INFINITY;
+      tmax = fmaxf(tmax, sacc[r]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float mnew = fmaxf(m, tmax);
+    // a query with no visible key so far keeps m = -inf: guard the exponentials
+    const float corr = mnew > -INFINITY ? __expf(m - mnew) : 1.f;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float pr = sacc[r] > -INFINITY ? __expf(sacc[r] - mnew) : 0.f;
+      sacc[r] = pr;
+      psum += pr;
+    }
+    lsum = lsum * corr + psum;
+    m = mnew;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { o0[r] *= corr; o1[r] *= corr; }
+    // O^T[dim][query] += sum_key V[key][dim] P[query][key]; step i visits the key of register i
+    {
+      const float* vr = Vs + hh * 4 * AHS + l32;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float* vk = vr + ((i >> 2) * 8 + (i & 3)) * AHS;
+        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vk[0], sacc[i], o0, 0, 0, 0);
+        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vk[32], sacc[i], o1, 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  lsum += __shfl_xor(lsum, 32);  // the two halves of a column saw disjoint keys, the same maximum
+
+  // merge of the four waves: each leaves O^T (64 x 32), m and l of its key run in its own LDS region
+  float* Om = am_lds + wave * AM_WAVE_FLOATS;  // [AHS][AMOST], then m[AMQ], l[AMQ]
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int dim = (r >> 2) * 8 + hh * 4 + (r & 3);
+    Om[dim * AMOST + l32] = o0[r];
+    Om[(dim + 32) * AMOST + l32] = o1[r];
+  }
+  if (hh == 0) {
+    Om[AHS * AMOST + l32] = m;
+    Om[AHS * AMOST + AMQ + l32] = lsum;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < AMQ * AHS / WG; ++j) {
+    const int e = tid + WG * j, qi = e >> 6, dim = e & 63;
+    float mw[NWAVE], M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) {
+      mw[w] = am_lds[w * AM_WAVE_FLOATS + AHS * AMOST + qi];
+      M = fmaxf(M, mw[w]);
+    }
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) {
+      const float f = mw[w] > -INFINITY ? __expf(mw[w] - M) : 0.f;
+      num += am_lds[w * AM_WAVE_FLOATS + dim * AMOST + qi] * f;
+      den += am_lds[w * AM_WAVE_FLOATS + AHS * AMOST + AMQ + qi] * f;
+    }
+    if (q0 + qi < Tq) out[(size_t)(q0 + qi) * ldo + h * AHS + dim] = num / den;
+  }
+}
+
 __global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* __restrict__ src, int lds,
                                                         float* __restrict__ dst, int ldd) {
   const int r = blockIdx.y;
@@ -931,6 +1089,19 @@ hipError_t launch_vocab_gemv(int V, int d, const float* x, const float* wte, flo
 
 hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const float* q, int ldq, const float* Kc,
                             const float* Vc, size_t hstride, int ldkv, float* out, int ldo, hipStream_t s) {
+  // a block of 32 queries per workgroup on the matrix cores
+  if (hs == AHS && Tq >= AMQ) {
+    static_assert(AHS * AMOST + 2 * AMQ <= AM_WAVE_FLOATS, "merge area must fit a wave's tile area");
+    const size_t lds = sizeof(float) * NWAVE * AM_WAVE_FLOATS;
+    static bool enabled = false;
+    if (!enabled) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      enabled = true;
+    }
+    attention_mfma_kernel<<<dim3(H, cdiv(Tq, AMQ)), WG, lds, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
+    return hipGetLastError();
+  }
   // enough (head, query block) workgroups to fill the GPU; else one workgroup per query row
   if (hs == AHS && Tq >= ATQ && H * cdiv(Tq, ATQ) >= 128) {
     attention_tile_kernel<<<dim3(H, cdiv(Tq, ATQ)), WG, 0, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
