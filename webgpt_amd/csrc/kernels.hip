@@ -656,7 +656,7 @@ __global__ __launch_bounds__(WG) void attention_tile_kernel(int Tq, int pos0, fl
 
 // ---------------------------------------------------------------------------
 // Prefill attention on the matrix cores (head size 64, at least 32 queries).
-// A workgroup owns 32 queries of one head; its four waves split the visible keys
+// A workgroup owns 32 queries of one head; its four or eight waves split the visible keys
 // into contiguous runs of 32-key tiles and are merged at the end (flash-decoding).
 // Everything is computed transposed, S^T = K Q^T and O^T = V^T P^T, with
 // v_mfma_f32_32x32x2_f32: an accumulator then holds, per lane, 16 keys (or output
@@ -678,7 +678,8 @@ constexpr int AMKST = AHS + 4; // row stride of a staged K tile (conflict-free 1
 constexpr int AM_WAVE_FLOATS = AMK * AMKST + AMK * AHS;  // K tile + V tile of one wave
 constexpr int AMOST = AMQ + 1; // row stride of a wave's O^T[dim][query] in the merge
 
-__global__ __launch_bounds__(WG) void attention_mfma_kernel(int Tq, int pos0, float scale, const float* __restrict__ q, int ldq,
+template <int NWV>
+__global__ __launch_bounds__(NWV * 64) void attention_mfma_kernel(int Tq, int pos0, float scale, const float* __restrict__ q, int ldq,
                                                              const float* __restrict__ Kc, const float* __restrict__ Vc,
                                                              size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
   extern __shared__ __attribute__((aligned(16))) float am_lds[];
@@ -694,7 +695,7 @@ __global__ __launch_bounds__(WG) void attention_mfma_kernel(int Tq, int pos0, fl
   const int qlast = q0 + AMQ - 1 < Tq - 1 ? q0 + AMQ - 1 : Tq - 1;
   const int nkeys = pos0 + qlast + 1;        // keys any query of the block sees
   const int nt = (nkeys + AMK - 1) / AMK;
-  const int per = (nt + NWAVE - 1) / NWAVE;
+  const int per = (nt + NWV - 1) / NWV;
   const int tb = wave * per;
   const int te = tb + per < nt ? tb + per : nt;
 
@@ -712,20 +713,32 @@ __global__ __launch_bounds__(WG) void attention_mfma_kernel(int Tq, int pos0, fl
 #pragma unroll
   for (int r = 0; r < 16; ++r) { o0[r] = 0.f; o1[r] = 0.f; }
 
-  for (int t = tb; t < te; ++t) {
+  // the tile after the current one is already on its way from memory while the current one is multiplied
+  float4 kreg[8], vreg[8];
+  auto fetch = [&](int t) {
     const int k0 = t * AMK;
-    // stage the K and V tiles of this wave: 32 rows x 16 float4 each, 8 per lane; rows past the end are zero
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int f = lane + 64 * j, row = f >> 4, c4 = f & 15;
-      float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), vv = kv;
-      if (k0 + row < nkeys) {
-        kv = ld4(kbase + (size_t)(k0 + row) * ldkv + 4 * c4);
-        vv = ld4(vbase + (size_t)(k0 + row) * ldkv + 4 * c4);
+      kreg[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      vreg[j] = kreg[j];
+      if (t < te && k0 + row < nkeys) {  // rows past the end are zero
+        kreg[j] = ld4(kbase + (size_t)(k0 + row) * ldkv + 4 * c4);
+        vreg[j] = ld4(vbase + (size_t)(k0 + row) * ldkv + 4 * c4);
       }
-      st4(Ks + row * AMKST + 4 * c4, kv);
-      st4(Vs + row * AHS + 4 * c4, vv);
     }
+  };
+  fetch(tb);
+  for (int t = tb; t < te; ++t) {
+    const int k0 = t * AMK;
+    // stage the K and V tiles of this wave: 32 rows x 16 float4 each, 8 per lane
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int f = lane + 64 * j, row = f >> 4, c4 = f & 15;
+      st4(Ks + row * AMKST + 4 * c4, kreg[j]);
+      st4(Vs + row * AHS + 4 * c4, vreg[j]);
+    }
+    fetch(t + 1);
     __builtin_amdgcn_wave_barrier();  // the tiles are private to the wave: LDS operations of a wave complete in order
     // S^T[key][query] = sum_dim K[key][dim] Q[query][dim]
     f32x16 sacc;
@@ -793,17 +806,17 @@ __global__ __launch_bounds__(WG) void attention_mfma_kernel(int Tq, int pos0, fl
   }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < AMQ * AHS / WG; ++j) {
-    const int e = tid + WG * j, qi = e >> 6, dim = e & 63;
-    float mw[NWAVE], M = -INFINITY;
+  for (int j = 0; j < AMQ * AHS / (NWV * 64); ++j) {
+    const int e = tid + NWV * 64 * j, qi = e >> 6, dim = e & 63;
+    float mw[NWV], M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NWAVE; ++w) {
+    for (int w = 0; w < NWV; ++w) {
       mw[w] = am_lds[w * AM_WAVE_FLOATS + AHS * AMOST + qi];
       M = fmaxf(M, mw[w]);
     }
     float num = 0.f, den = 0.f;
 #pragma unroll
-    for (int w = 0; w < NWAVE; ++w) {
+    for (int w = 0; w < NWV; ++w) {
       const float f = mw[w] > -INFINITY ? __expf(mw[w] - M) : 0.f;
       num += am_lds[w * AM_WAVE_FLOATS + dim * AMOST + qi] * f;
       den += am_lds[w * AM_WAVE_FLOATS + AHS * AMOST + AMQ + qi] * f;
@@ -1092,14 +1105,21 @@ hipError_t launch_attention(int Tq, int pos0, int H, int hs, float scale, const 
   // a block of 32 queries per workgroup on the matrix cores
   if (hs == AHS && Tq >= AMQ) {
     static_assert(AHS * AMOST + 2 * AMQ <= AM_WAVE_FLOATS, "merge area must fit a wave's tile area");
-    const size_t lds = sizeof(float) * NWAVE * AM_WAVE_FLOATS;
+    // eight waves once the longest query block has more than eight key tiles
+    const bool wide = cdiv(pos0 + Tq, AMK) > 8;
+    const size_t lds = sizeof(float) * (wide ? 8 : 4) * AM_WAVE_FLOATS;
     static bool enabled = false;
     if (!enabled) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)(sizeof(float) * 4 * AM_WAVE_FLOATS));
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)(sizeof(float) * 8 * AM_WAVE_FLOATS));
       if (e != hipSuccess) return e;
       enabled = true;
     }
-    attention_mfma_kernel<<<dim3(H, cdiv(Tq, AMQ)), WG, lds, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
+    if (wide) attention_mfma_kernel<8><<<dim3(H, cdiv(Tq, AMQ)), 512, lds, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
+    else attention_mfma_kernel<4><<<dim3(H, cdiv(Tq, AMQ)), 256, lds, s>>>(Tq, pos0, scale, q, ldq, Kc, Vc, hstride, ldkv, out, ldo);
     return hipGetLastError();
   }
   // enough (head, query block) workgroups to fill the GPU; else one workgroup per query row
