@@ -341,22 +341,28 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
   for (int k0 = kbeg; k0 < kend; k0 += BK) {
     const bool more = k0 + BK < kend;
     if (more) fetch(k0 + BK);
+    // QS quarter-steps of operands are read from LDS at a time, then their matrix instructions run
+    // back to back: the whole step for the small tile (32 registers), a quarter for the large one
+    constexpr int QS = RB * CB == 1 ? HK / 4 : 1;
 #pragma unroll
-    for (int q = 0; q < HK / 4; ++q) {  // four instructions per block and quarter-step: one 128-bit A read each
-      float av[RB][4], bv[CB][4];
+    for (int q0 = 0; q0 < HK / 4; q0 += QS) {
+      float av[RB][4 * QS], bv[CB][4 * QS];
 #pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + q * 4);
-        av[r][0] = v.x; av[r][1] = v.y; av[r][2] = v.z; av[r][3] = v.w;
+      for (int q = 0; q < QS; ++q) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+          const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + (q0 + q) * 4);
+          av[r][4 * q] = v.x; av[r][4 * q + 1] = v.y; av[r][4 * q + 2] = v.z; av[r][4 * q + 3] = v.w;
+        }
+#pragma unroll
+        for (int c = 0; c < CB; ++c) {
+          const float* bp = Bs[st] + (h + 8 * (q0 + q)) * TN + wn + c * 32 + l32;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) bv[c][4 * q + i] = bp[2 * i * TN];
+        }
       }
 #pragma unroll
-      for (int c = 0; c < CB; ++c) {
-        const float* bp = Bs[st] + (h + 8 * q) * TN + wn + c * 32 + l32;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) bv[c][i] = bp[2 * i * TN];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4 * QS; ++i)
 #pragma unroll
         for (int r = 0; r < RB; ++r)
 #pragma unroll
