@@ -31,7 +31,7 @@ def run(inst, shape):
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 4), (1, 768, 768), (1, 2304, 768), (1, 768, 3072), (1, 72, 100), (2, 64, 64),
                                    (3, 1600, 1600), (4, 384, 1536), (5, 8, 12), (7, 200, 36), (16, 768, 768),
-                                   (128, 2304, 768), (65, 136, 260), (200, 768, 3072)])
+                                   (128, 2304, 768), (65, 136, 260), (200, 768, 3072), (2048, 4096, 64), (2050, 4104, 40)])
 def test_fast_matmul(device, M, N, K):
     A, W, b = rnd(M, K), rnd(K, N, scale=0.05), rnd(N)
     inst = FastMatMulBlock.newInstance(M, N, K, init_tensor(A, [M, K]), init_tensor(W, [K, N]), init_tensor(b, [N]))
@@ -110,7 +110,7 @@ def test_deembed_ragged_vocab(device):
     assert close(got, want), worst(got, want)
 
 
-@pytest.mark.parametrize("T,H,hs", [(1, 2, 8), (15, 4, 32), (64, 6, 64), (130, 12, 64), (5, 2, 4), (33, 25, 64)])
+@pytest.mark.parametrize("T,H,hs", [(1, 2, 8), (15, 4, 32), (64, 6, 64), (130, 12, 64), (5, 2, 4), (33, 25, 64), (20, 3, 64), (300, 2, 64)])
 def test_attention(device, T, H, hs):
     d = H * hs
     x = rnd(T, d)
