@@ -15,10 +15,10 @@ constexpr int PD_SPLIT = 4;      // position slices per head in the attention ph
 constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
-// [w*cpw, (w+1)*cpw) of N; a column is S segments of 256 contraction elements; the
-// cpw*S items of a workgroup are dealt to its waves in runs of ipw.
+// [w*cpw, (w+1)*cpw) of N; a column is S segments ("items") of 256 contraction elements,
+// stored column by column.
 struct PhaseGeom {
-  int N, cpw, S, ipw;
+  int N, cpw, S;
 };
 
 // Offsets (in floats) inside one layer's block of small parameters:

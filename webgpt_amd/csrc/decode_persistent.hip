@@ -9,8 +9,9 @@
 //   - every linear layer is split by output columns over the workgroups; a
 //     workgroup's share of W is a contiguous slab laid out at load time so that
 //     each wave reads 1 KB per instruction (float4 per lane);
-//   - the slab of a phase is requested into registers two phases ahead, so HBM
-//     streams continuously while the dependent arithmetic of earlier phases runs;
+//   - the slab of a phase is requested into registers a phase ahead (right after the
+//     poll that starts the phase before it, where two register sets fit), so it
+//     lands while that phase computes and never queues in front of a poll;
 //   - phases exchange their (small) output vectors through global memory as
 //     {value, epoch} 64-bit words written and polled with device-scope relaxed
 //     atomics: the epoch makes each word self-validating, so no barrier and no
@@ -23,7 +24,8 @@
 //     finishes redundantly, so the next token needs no broadcast hop.
 //
 // Every wait is bounded: a poll that does not complete within SPIN_LIMIT rounds
-// raises the error word and the workgroup leaves; all others then follow.
+// raises the error word; every later wait of every workgroup then ends at once and
+// the launch drains.
 #include "decode_persistent.h"
 
 #include <cstdio>
@@ -34,9 +36,6 @@ namespace wgpt {
 namespace {
 
 typedef unsigned long long u64;
-#ifndef WGPT_DBG_SKIP_W
-#define WGPT_DBG_SKIP_W 0
-#endif
 
 constexpr int NT = PD_THREADS;       // threads per workgroup
 constexpr int NW = NT / 64;          // waves per workgroup
@@ -317,11 +316,7 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
     float sum = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) sum += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
-#ifdef WGPT_DBG_NOSTATS
-    const float mean = sum * 1e-30f;
-#else
     const float mean = wave_sum(sum) * (1.0f / (float)K);
-#endif
     float q = 0.f;
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
@@ -331,11 +326,7 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
       const float qq = (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
       q += in ? qq : 0.f;
     }
-#ifdef WGPT_DBG_NOSTATS
-    const float rstd = 1.0f + q * 1e-30f;
-#else
     const float rstd = fast_rsqrt(wave_sum(q) * (1.0f / (float)K) + 1e-5f);
-#endif
 #pragma unroll
     for (int s2 = 0; s2 < S; ++s2) {
       const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
@@ -474,10 +465,7 @@ struct Phases {
   // Two register sets (c_attn and c_fc in one, the two projections in the other) let a
   // phase's weights be requested a whole phase ahead, right after the poll of the
   // phase before it; affordable while a set is at most 32 registers.
-#ifndef WGPT_DUAL_LIMIT
-#define WGPT_DUAL_LIMIT 32
-#endif
-  static constexpr bool DUAL = MAXI * (C::I8 ? 1 : 4) <= WGPT_DUAL_LIMIT;
+  static constexpr bool DUAL = MAXI * (C::I8 ? 1 : 4) <= 32;
 };
 
 template <class C, int MAXKV>
@@ -784,13 +772,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
         const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane);
         TRACE5(2);
-        if (finD) 
-#ifdef WGPT_DBG_NOGELU
-          pubD[fc] = finish<I8>(dot, wX) * 0.01f;
-#else
-          pubD[fc] = gelu_ref(finish<I8>(dot, wX));
-#endif
-  // model.js:188
+        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, wX));  // model.js:188
         __syncthreads();
         ++ep;
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
@@ -1022,7 +1004,6 @@ PhaseGeom make_geom(int N, int K) {
   g.N = N;
   g.cpw = (N + PD_GRID - 1) / PD_GRID;
   g.S = (K + SEG - 1) / SEG;
-  g.ipw = (g.cpw * g.S + NW - 1) / NW;
   return g;
 }
 
