@@ -217,3 +217,25 @@ def test_int8_persistent_decode_against_oracle(device):
         assert close(out[mode][-1], want), (mode, worst(out[mode][-1], want))
     assert greedy_ok(out[1][-1], want)
     gpt.unloadBuffers()
+
+
+def test_expired_wait_disables_the_persistent_path_and_falls_back(device, monkeypatch):
+    """A bounded wait of the persistent kernel that expires (forced from the host by a poll limit of
+    one round: every workgroup gives up at once and the launch drains normally) is reported as an
+    error, and decoding continues on the per-block kernels with correct results."""
+    cfg = small_cfg(n_layer=2, n_head=6, n_embd=384, n_ctx=32, vocab_size=90)
+    monkeypatch.setenv("WEBGPT_AMD_SPIN_LIMIT", "1")
+    gpt, tensors = load(cfg, seed=17)
+    monkeypatch.delenv("WEBGPT_AMD_SPIN_LIMIT")
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(17, "prompt", 10, cfg["vocab_size"])
+    gpt.prefill(tokens[:8])
+    with pytest.raises(WgptError, match="bounded wait expired"):
+        gpt.decode(int(tokens[8]))
+    with pytest.raises(WgptError, match="not available"):
+        gpt.set_decode_mode(1)
+    got = gpt.decode(int(tokens[8]))                  # same token again, now on the per-block path
+    assert close(got, ref.forward(p, w, tokens[:9])), worst(got, ref.forward(p, w, tokens[:9]))
+    got = gpt.decode(int(tokens[9]))
+    assert close(got, ref.forward(p, w, tokens[:10]))
+    gpt.unloadBuffers()

@@ -62,6 +62,7 @@ struct PersistentArgs {
   // [2] attention outputs on the attention workgroups, [3] on the others,
   // [4] residual row into c_fc, [5] hidden row, [6] arg-max candidates
   int delay[7];
+  unsigned spin_limit;  // poll rounds after which a wait gives up and raises *err
   unsigned ebase;      // epoch of the last word published by earlier launches
   int pos0, nsteps;
 };

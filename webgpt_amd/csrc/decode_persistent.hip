@@ -23,7 +23,7 @@
 //     contraction index), followed by a distributed arg-max that every workgroup
 //     finishes redundantly, so the next token needs no broadcast hop.
 //
-// Every wait is bounded: a poll that does not complete within SPIN_LIMIT rounds
+// Every wait is bounded: a poll that does not complete within `spin_limit` rounds
 // raises the error word; every later wait of every workgroup then ends at once and
 // the launch drains.
 #include "decode_persistent.h"
@@ -40,7 +40,6 @@ typedef unsigned long long u64;
 constexpr int NT = PD_THREADS;       // threads per workgroup
 constexpr int NW = NT / 64;          // waves per workgroup
 constexpr int SEG = 256;             // contraction elements per item (64 lanes x float4)
-constexpr unsigned SPIN_LIMIT = 1u << 18;
 
 __device__ __forceinline__ u64 ld_word(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_word(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -168,7 +167,8 @@ __device__ __forceinline__ void nap(int units) {
 }
 
 template <int N>
-__device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err, int delay) {
+__device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err, int delay,
+                                           unsigned spin_limit) {
   constexpr int NP = (N + NT - 1) / NT;
   const int t = opaque(threadIdx.x);
   unsigned pending = 0;
@@ -190,7 +190,7 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
       }
     if (pending) {
       ++spins;
-      if (spins > SPIN_LIMIT || bail_flag() ||
+      if (spins > spin_limit || bail_flag() ||
           ((spins & 255u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
         sh.bail = 1;
         atomicCAS(err, 0, (int)epoch);
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       {
         [[maybe_unused]] constexpr int PH = PH_QKV;
         if (li > 0) {
-          poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0]);
+          poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0], a.spin_limit);
           if (!FOLD) deposit_ln<D>(lnreg, lnp);
           __syncthreads();
           if (sh.bail) return;
@@ -623,7 +623,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
             if ((unsigned)(pk >> 32) == ep - 1) {
               qkv_s[tid] = __uint_as_float((unsigned)pk);
               pending = 0;
-            } else if (++spins > SPIN_LIMIT || bail_flag()) {
+            } else if (++spins > a.spin_limit || bail_flag()) {
               sh.bail = 1;
               atomicCAS(a.err, 0, (int)ep);
               break;
@@ -708,7 +708,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
         [[maybe_unused]] constexpr int PH = PH_PROJ;
-        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3]);
+        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -764,7 +764,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= c_fc: LN2 + fc + GELU =======================
       {
         [[maybe_unused]] constexpr int PH = PH_FC;
-        poll_words<D>(a.bufR1, ep, xs0, a.err, a.delay[4]);
+        poll_words<D>(a.bufR1, ep, xs0, a.err, a.delay[4], a.spin_limit);
         if (!FOLD) deposit_ln<D>(lnreg, lnp);
         __syncthreads();
         wait_loads();
@@ -796,7 +796,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
             if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
           }
         };
-        poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5]);
+        poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -816,7 +816,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
 
     // ======================= final LayerNorm + vocabulary projection =======================
-    poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0]);
+    poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0], a.spin_limit);
     if (!FOLD) deposit_ln<D>(lnreg, lnp);
     __syncthreads();
     if (sh.bail) return;
@@ -886,7 +886,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
-    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err, a.delay[6]);
+    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err, a.delay[6], a.spin_limit);
     if (!FOLD && step + 1 < a.nsteps) deposit_ln<D>(lnreg, lnp);  // every wave is past the final LayerNorm: the arg-max words need all of them
     __syncthreads();
     if (sh.bail) return;

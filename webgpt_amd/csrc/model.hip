@@ -278,6 +278,13 @@ static int setup_persistent(Model* m) {
         for (int i = 0; i < 7; ++i) a.delay[i] = v[i] < 0 ? 0 : (v[i] > 1024 ? 1024 : v[i]);
     }
   }
+  // a wait that takes this many poll rounds (a quarter of a second) means a workgroup is not running;
+  // WEBGPT_AMD_SPIN_LIMIT lowers it (tests of the fallback force an expiry this way)
+  a.spin_limit = 1u << 18;
+  if (const char* e = getenv("WEBGPT_AMD_SPIN_LIMIT")) {
+    const long v = atol(e);
+    if (v >= 1 && v < (1l << 30)) a.spin_limit = (unsigned)v;
+  }
   a.trace = nullptr;
 #ifdef WGPT_TRACE
   // Profiling builds: per-workgroup clock samples of the last step of each launch.
