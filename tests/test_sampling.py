@@ -26,7 +26,7 @@ def cases():
     rng = np.random.default_rng(11)
     out = []
     for V, k, T in ((1, 1, 1.0), (5, 3, 1.0), (5, 9, 0.5), (65, 2, 1.0), (1000, 40, 0.7), (50257, 1, 1.0), (50257, 3, 1.0),
-                    (50257, 50, 1.3), (4099, 1024, 2.0)):
+                    (50257, 50, 1.3), (4099, 1024, 2.0), (70001, 5, 1.0)):
         x = (rng.standard_normal(V) * 3).astype(np.float32)
         if V > 4:
             x[rng.integers(0, V, 6)] = x.max() + 1.0      # ties at the top: the lowest index must come first

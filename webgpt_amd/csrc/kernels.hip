@@ -864,6 +864,9 @@ __device__ __forceinline__ bool better(float ov, int oi, float cv, int ci) {
   return oi != 0x7fffffff && (ci == 0x7fffffff || ov > cv || (ov == cv && oi < ci));
 }
 
+// REG: the logits of a thread's stride (V <= 65536: at most 64 of them) stay in registers, so the
+// owner's search for its next candidate after a selection touches no memory.
+template <bool REG>
 __global__ __launch_bounds__(1024) void sample_topk_kernel(int V, int k, double temperature, const double* __restrict__ u,
                                                             const float* __restrict__ logits, int32_t* tok, int32_t* out, int slot,
                                                             int32_t* ids, double* probs) {
@@ -874,12 +877,30 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(int V, int k, double 
   __shared__ int sel_i[SAMPLE_MAX_K];
   __shared__ double ev[SAMPLE_MAX_K];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < (V + 31) / 32; i += 1024) taken[i] = 0u;
+  if (!REG)
+    for (int i = tid; i < (V + 31) / 32; i += 1024) taken[i] = 0u;
   if (k > V) k = V;
+  float mine[REG ? 64 : 1];
+  unsigned long long gone = 0ull;  // REG: bit j set once element tid + 1024 j has been selected
+  if (REG) {
+#pragma unroll
+    for (int j = 0; j < 64; ++j) mine[j] = tid + 1024 * j < V ? logits[tid + 1024 * j] : -INFINITY;
+  }
   // this thread's candidate: the best not yet taken element of its stride
   auto scan = [&](float& best, int& besti) {
     best = -INFINITY;
     besti = 0x7fffffff;
+    if (REG) {
+#pragma unroll
+      for (int j = 0; j < 64; ++j) {
+        const int i = tid + 1024 * j;
+        if (i < V && !((gone >> j) & 1ull) && (mine[REG ? j : 0] > best || besti == 0x7fffffff)) {
+          best = mine[REG ? j : 0];
+          besti = i;
+        }
+      }
+      return;
+    }
     for (int i = tid; i < V; i += 1024) {
       if (taken[i >> 5] & (1u << (i & 31))) continue;
       const float v = logits[i];
@@ -924,7 +945,8 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(int V, int k, double 
       sel_i[r] = ci;
     }
     if ((ci & 1023) == tid) {
-      taken[ci >> 5] |= 1u << (ci & 31);
+      if (REG) gone |= 1ull << (ci >> 10);
+      else taken[ci >> 5] |= 1u << (ci & 31);
       scan(best, besti);
     }
     __syncthreads();
@@ -1155,7 +1177,8 @@ hipError_t launch_kv_append(int T, int d, int hs, int ctx, int pos0, const float
 hipError_t launch_sample_topk(int V, int k, double temperature, const double* u, const float* logits, int32_t* tok,
                               int32_t* out, int slot, int32_t* ids, double* probs, hipStream_t s) {
   if (V < 1 || V > SAMPLE_MAX_V || k < 1 || k > SAMPLE_MAX_K) return hipErrorInvalidValue;
-  sample_topk_kernel<<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
+  if (V <= 65536) sample_topk_kernel<true><<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
+  else sample_topk_kernel<false><<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
   return hipGetLastError();
 }
 
