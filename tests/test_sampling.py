@@ -90,9 +90,11 @@ def test_device_selection_rejects_bad_arguments(device):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("mode", [0, 1])
-def test_decode_sample_follows_the_reference_loop(device, mode):
-    """wgpt_decode_sample == per token: logits of the window (oracle), then model.js:81-85."""
+@pytest.mark.parametrize("mode,top_k", [(0, 5), (1, 2), (1, 5), (1, 8), (1, 9)])
+def test_decode_sample_follows_the_reference_loop(device, mode, top_k):
+    """wgpt_decode_sample == per token: logits of the window (oracle), then model.js:81-85.
+    Mode 1 selects and samples inside the persistent kernel up to top_k = 8 and per token with the
+    selection kernel above that."""
     from oracle import ref
     from webgpt_amd.model import GPT
     cfg = small_cfg(n_layer=2, n_head=6, n_embd=384, n_ctx=48, vocab_size=300)
@@ -108,7 +110,7 @@ def test_decode_sample_follows_the_reference_loop(device, mode):
         prompt = [int(t) for t in synth.tokens(21, "prompt", 10, cfg["vocab_size"])]
         rng = np.random.default_rng(5)
         u = rng.random(12)
-        top_k, T = 5, 0.8
+        T = 0.8
         lg = gpt.prefill(prompt)
         first, _, _ = ref.sample_topk(lg, top_k, T, 0.5)
         got = gpt.decode_sample(first, len(u), top_k, T, u)

@@ -12,6 +12,7 @@ namespace wgpt {
 constexpr int PD_THREADS = 512;  // threads per workgroup
 constexpr int PD_GRID = 256;     // workgroups: one per compute unit of an MI355X
 constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase
+constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
 constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
@@ -63,6 +64,11 @@ struct PersistentArgs {
   // [4] residual row into c_fc, [5] hidden row, [6] arg-max candidates
   int delay[7];
   unsigned spin_limit;  // poll rounds after which a wait gives up and raises *err
+  // token selection: top_k == 1 is the arg-max; 2..PD_TOPK samples as GPT.generate does
+  // (model.js:81-85) with u[step] for the step's Math.random() and the float64 temperature
+  int top_k;
+  double temperature;
+  const double* u;  // [nsteps], device memory (unused for top_k == 1)
   unsigned ebase;      // epoch of the last word published by earlier launches
   int pos0, nsteps;
 };

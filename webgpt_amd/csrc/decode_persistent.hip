@@ -115,6 +115,8 @@ struct Shared {
   int bail;
   float red[32];
   float red_idx[NW];
+  float cand_v[NW * PD_TOPK];  // per-wave top-k candidates of the vocabulary phase
+  int cand_i[NW * PD_TOPK];
 };
 __shared__ Shared sh;
 
@@ -450,6 +452,25 @@ __device__ __forceinline__ float finish(float dot, const WS& ws) {
 #define TRACE5(k) do {} while (0)
 #endif
 
+// Order of selectTopK (globals.js:66-74): larger logit first, lower index first among equals;
+// index INT_MAX marks an empty candidate.
+constexpr int NOCAND = 0x7fffffff;
+__device__ __forceinline__ bool cand_before(float ov, int oi, float cv, int ci) {
+  return oi != NOCAND && (ci == NOCAND || ov > cv || (ov == cv && oi < ci));
+}
+// The first candidate of the wave in that order, as wave-uniform values.
+__device__ __forceinline__ void wave_first(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off);
+    const int oi = __shfl_xor(i, off);
+    if (cand_before(ov, oi, v, i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
 // Linear phases of a layer, in execution order.
 enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
 
@@ -468,7 +489,9 @@ struct Phases {
   static constexpr bool DUAL = MAXI * (C::I8 ? 1 : 4) <= 32;
 };
 
-template <class C, int MAXKV>
+// SAMPLE: top-k selection and sampling in the kernel (top_k in 2..PD_TOPK); the arg-max kernel
+// stays free of its registers.
+template <class C, int MAXKV, bool SAMPLE>
 __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a) {
   typedef Phases<C> PS;
   typedef typename PS::A PA;
@@ -480,7 +503,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
-  constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;     // floats of the staged exchange words
+  constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;  // floats of the staged exchange words
   constexpr int PART = 32 * (HS + 4) > PE::CPW * NW ? 32 * (HS + 4) : PE::CPW * NW;
   constexpr int NLN = (D / 2 + NT - 1) / NT;                        // float4 of LayerNorm parameters per thread
 
@@ -833,6 +856,16 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       input_row<D, true, true>(xv, xs0, lnp, lane);
       float best = -INFINITY;
       int besti = 0x7fffffff;
+      // top_k > 1: this wave's K best rows so far, in order; (lastv, lasti) is the K-th
+      const int K = SAMPLE ? a.top_k : 1;
+      constexpr int KL = SAMPLE ? PD_TOPK : 1;
+      float tv[KL], lastv = -INFINITY;
+      int ti[KL], lasti = NOCAND;
+#pragma unroll
+      for (int j = 0; j < KL; ++j) {
+        tv[j] = -INFINITY;
+        ti[j] = NOCAND;
+      }
       for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
         float4 w[R][S];
 #pragma unroll
@@ -856,6 +889,26 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
               best = s;
               besti = vb + r;
             }
+            if (SAMPLE && cand_before(s, vb + r, lastv, lasti)) {
+              // insert: carry the displaced candidate down the list
+              float cv = s;
+              int ci = vb + r;
+#pragma unroll
+              for (int j = 0; j < KL; ++j) {
+                if (j < K && cand_before(cv, ci, tv[j], ti[j])) {
+                  const float sv = tv[j];
+                  const int si = ti[j];
+                  tv[j] = cv;
+                  ti[j] = ci;
+                  cv = sv;
+                  ci = si;
+                }
+                if (j == K - 1) {
+                  lastv = tv[j];
+                  lasti = ti[j];
+                }
+              }
+            }
           }
         }
       }
@@ -863,9 +916,46 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         sh.red[wave] = best;
         sh.red_idx[wave] = __int_as_float(besti);
       }
+      if (SAMPLE && lane < PD_TOPK) {
+        float cvv = -INFINITY;
+        int cii = NOCAND;
+#pragma unroll
+        for (int j = 0; j < KL; ++j)
+          if (lane == j) {
+            cvv = tv[j];
+            cii = ti[j];
+          }
+        sh.cand_v[wave * PD_TOPK + lane] = cvv;
+        sh.cand_i[wave * PD_TOPK + lane] = cii;
+      }
       __syncthreads();
       ++ep;
-      if (tid == 0) {
+      if (SAMPLE) {
+        // the workgroup's K best of its waves' candidates (one per lane of wave 0), published in order
+        if (wave == 0) {
+          float cv = sh.cand_v[lane];
+          int ci = sh.cand_i[lane];
+          float wv = -INFINITY;
+          int wi = NOCAND;
+          for (int r = 0; r < K; ++r) {
+            float fv = cv;
+            int fi = ci;
+            wave_first(fv, fi);
+            if (lane == r) {
+              wv = fv;
+              wi = fi;
+            }
+            if (ci == fi) {  // indices are unique: the owner retires its candidate
+              cv = -INFINITY;
+              ci = NOCAND;
+            }
+          }
+          if (lane < PD_TOPK) {
+            publish(a.bufAM + 2 * (wg * PD_TOPK + lane), wv, ep);
+            publish(a.bufAM + 2 * (wg * PD_TOPK + lane) + 1, __int_as_float(wi), ep);
+          }
+        }
+      } else if (tid == 0) {
         float b = sh.red[0];
         int bi = __float_as_int(sh.red_idx[0]);
         for (int v = 1; v < NW; ++v) {
@@ -886,12 +976,77 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
-    poll_words<2 * C::G>(a.bufAM, ep, attp, a.err, a.delay[6], a.spin_limit);
+    double ustep = 0.0;
+    if (SAMPLE) {
+      ustep = a.u[step];
+      poll_words<2 * PD_TOPK * C::G>(a.bufAM, ep, attp, a.err, a.delay[6], a.spin_limit);
+    } else {
+      poll_words<2 * C::G>(a.bufAM, ep, attp, a.err, a.delay[6], a.spin_limit);
+    }
     if (!FOLD && step + 1 < a.nsteps) deposit_ln<D>(lnreg, lnp);  // every wave is past the final LayerNorm: the arg-max words need all of them
     __syncthreads();
     if (sh.bail) return;
     TRACE(3 + a.L * 8);
-    {
+    if (SAMPLE) {
+      // Every wave of every workgroup selects the same K candidates in order (selectTopK), applies
+      // cpuSoftmax in float64 and sampleFromDistribution with the step's draw (globals.js:47-74).
+      // A workgroup's list arrives in order, so a lane only ever looks at the heads of its G/64 lists.
+      const int K = a.top_k;
+      constexpr int LPL = C::G / 64;  // workgroup lists per lane
+      static_assert(C::G % 64 == 0, "workgroup lists are dealt to lanes evenly");
+      float hv[LPL];
+      int hi[LPL], hp[LPL];
+#pragma unroll
+      for (int jj = 0; jj < LPL; ++jj) {
+        const int c = (lane + 64 * jj) * PD_TOPK;
+        hp[jj] = 0;
+        hv[jj] = attp[2 * c];
+        hi[jj] = __float_as_int(attp[2 * c + 1]);
+      }
+      float myv = -INFINITY;  // lane r keeps the r-th selection
+      int myi = NOCAND;
+      for (int r = 0; r < K; ++r) {
+        float fv = -INFINITY;
+        int fi = NOCAND;
+#pragma unroll
+        for (int jj = 0; jj < LPL; ++jj)
+          if (cand_before(hv[jj], hi[jj], fv, fi)) {
+            fv = hv[jj];
+            fi = hi[jj];
+          }
+        wave_first(fv, fi);
+        if (lane == r) {
+          myv = fv;
+          myi = fi;
+        }
+        // the owner moves on to the next entry of that list
+#pragma unroll
+        for (int jj = 0; jj < LPL; ++jj)
+          if (hi[jj] == fi && fi != NOCAND) {
+            ++hp[jj];
+            const int c = (lane + 64 * jj) * PD_TOPK + hp[jj];
+            hv[jj] = hp[jj] < K ? attp[2 * c] : -INFINITY;
+            hi[jj] = hp[jj] < K ? __float_as_int(attp[2 * c + 1]) : NOCAND;
+          }
+      }
+      // lane r: exp((x_r - max) / temperature); then the sums in the reference's order on every lane
+      const float first = __shfl(myv, 0);
+      const double mye = myi != NOCAND ? exp(((double)myv - (double)first) / a.temperature) : 0.0;
+      double sum = 0.0;
+      for (int r = 0; r < K; ++r) sum = sum + __shfl(mye, r);
+      double cum = 0.0;
+      int pick = NOCAND, lastsel = 0;
+      for (int r = 0; r < K; ++r) {
+        const int si = __shfl(myi, r);
+        if (si != NOCAND) {
+          cum += __shfl(mye, r) / sum;
+          lastsel = si;
+          if (pick == NOCAND && ustep < cum) pick = si;
+        }
+      }
+      tok = pick != NOCAND ? pick : lastsel;
+      if (wg == 0 && tid == 0) a.out_tok[step] = tok;
+    } else {
       float b = -INFINITY;
       int bi = 0x7fffffff;
       for (int w2 = lane; w2 < C::G; w2 += 64) {
@@ -975,7 +1130,7 @@ template <class C>
 size_t lds_bytes_of() {
   typedef Phases<C> PS;
   constexpr int XS = (C::SD + C::SH) * SEG;
-  constexpr int ATTP = C::ATTW > 2 * C::G ? C::ATTW : 2 * C::G;
+  constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;
   constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
   const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + 16);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
@@ -985,15 +1140,19 @@ size_t lds_bytes_of() {
 
 template <class C>
 hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
-  auto kern = decode_persistent_kernel<C, PD_MAXKV>;
   const size_t lds_bytes = lds_bytes_of<C>();
-  static bool enabled = false;  // dynamic LDS size already raised for this instantiation
+  static bool enabled = false;  // dynamic LDS size already raised for the two instantiations
   if (!enabled) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, PD_MAXKV, false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, PD_MAXKV, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
     enabled = true;
   }
-  kern<<<PD_GRID, NT, lds_bytes, s>>>(a);
+  if (a.top_k > 1) decode_persistent_kernel<C, PD_MAXKV, true><<<PD_GRID, NT, lds_bytes, s>>>(a);
+  else decode_persistent_kernel<C, PD_MAXKV, false><<<PD_GRID, NT, lds_bytes, s>>>(a);
   return hipGetLastError();
 }
 
@@ -1034,7 +1193,7 @@ bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
 }
 
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
-  if (!persistent_supports(a.d, a.H, a.ctx, a.weight_dtype)) return hipErrorInvalidValue;
+  if (!persistent_supports(a.d, a.H, a.ctx, a.weight_dtype) || a.top_k < 1 || a.top_k > PD_TOPK) return hipErrorInvalidValue;
   if (a.weight_dtype == 1) return launch_t<Shape<1600, 25, true>>(a, s);
   switch (a.d) {
     case 384: return launch_t<Shape<384, 6>>(a, s);

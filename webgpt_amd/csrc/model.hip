@@ -246,7 +246,7 @@ static int setup_persistent(Model* m) {
   a.lparams = lparams;
   a.wte = m->wte; a.wpe = m->wpe; a.lnf_g = m->lnf_g; a.lnf_b = m->lnf_b;
   a.kv = m->kv;
-  const size_t words = (size_t)3 * d + attw + d + hid + d + 2 * G;
+  const size_t words = (size_t)3 * d + attw + d + hid + d + 2 * PD_TOPK * G;
   unsigned long long* buf;
   if ((rc = dev_alloc(m, words * sizeof(unsigned long long), (void**)&buf))) return rc;
   WGPT_HIP(hipMemsetAsync(buf, 0, words * sizeof(unsigned long long), rt().stream));
@@ -298,12 +298,16 @@ static int setup_persistent(Model* m) {
 
 // Runs `steps` greedy decode steps from position m->pos with the persistent kernel.
 // The first token is in m->tok_dev[0]; chosen ids land in m->out_tok_dev.
-static int decode_persistent(Model* m, int steps) {
+// top_k == 1: greedy. Otherwise u_dev holds the steps' uniform draws.
+static int decode_persistent(Model* m, int steps, int top_k = 1, double temperature = 1.0, const double* u_dev = nullptr) {
   PersistentArgs a = m->pa;
+  a.top_k = top_k;
+  a.temperature = temperature;
+  a.u = u_dev;
   const unsigned per_step = persistent_epochs_per_step(m->L);
   if (m->epoch > 0xffffffffu - per_step * (unsigned)steps - 8u) {
     // epoch counter about to wrap: start over from clean exchange buffers
-    const size_t words = (size_t)(a.bufAM + 2 * PD_GRID - a.bufQKV);
+    const size_t words = (size_t)(a.bufAM + 2 * PD_TOPK * PD_GRID - a.bufQKV);
     WGPT_HIP(hipMemsetAsync(a.bufQKV, 0, words * sizeof(unsigned long long), rt().stream));
     m->epoch = 0;
   }
@@ -553,15 +557,23 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   const bool persistent = m->decode_mode == 1;
   const int k = top_k < m->V ? top_k : m->V;
-  for (int i = 0; i < steps; ++i) {
-    // one token per launch: the sampled id in tok_dev[0] is the next launch's input
-    int rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+  // up to PD_TOPK candidates the persistent kernel selects and samples itself, all steps in one launch
+  const bool in_kernel = persistent && k <= PD_TOPK;
+  if (in_kernel) {
+    int rc = decode_persistent(m, steps, k, temperature, m->u_dev);
     if (rc) return rc;
-    LAUNCH(launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream));
-    m->pos += 1;
+    m->pos += steps;
+  } else {
+    for (int i = 0; i < steps; ++i) {
+      // one token per launch: the sampled id in tok_dev[0] is the next launch's input
+      int rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+      if (rc) return rc;
+      LAUNCH(launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream));
+      m->pos += 1;
+    }
   }
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
-  WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
+  WGPT_HIP(hipMemcpyAsync(out_tokens, in_kernel ? m->out_tok_dev : m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
   if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
