@@ -83,12 +83,22 @@ class GPT {
     for (let i = 0; i < max_new_tokens; i++) {
       const idx_cond = history.slice(-this.params.n_ctx);
       const startTime = performance.now();
-      const logits = await this.run(idx_cond);
+      let idx_next;
+      const h = this._history;
+      const cached = h.length > 0 && idx_cond.length === h.length + 1 && idx_cond.length <= this.params.n_ctx && h.every((t, j) => t === idx_cond[j]);
+      if (cached && top_k >= 1 && top_k <= 1024 && temperature > 0) {
+        // the window extends the cached one by a token: that token goes in, the next one is selected
+        // on the device (selectTopK, cpuSoftmax, sampleFromDistribution with this Math.random() draw)
+        // and the logits are never read back
+        idx_next = this.decodeSample(idx_cond[idx_cond.length - 1], top_k, temperature, [Math.random()])[0];
+      } else {
+        const logits = await this.run(idx_cond);
+        const { topKIndices, topKProbs } = G.selectTopK(logits, top_k);
+        const probs = G.cpuSoftmax(topKProbs, temperature);
+        idx_next = topKIndices[G.sampleFromDistribution(probs)];
+      }
       const lapsedTime = performance.now() - startTime;
       i >= warmupRuns && (totalTime += lapsedTime);
-      const { topKIndices, topKProbs } = G.selectTopK(logits, top_k);
-      const probs = G.cpuSoftmax(topKProbs, temperature);
-      const idx_next = topKIndices[G.sampleFromDistribution(probs)];
       history = history.concat(idx_next);
       yield this.tokenizer ? this.tokenizer.decode([idx_next]) : idx_next;
     }

@@ -16,6 +16,7 @@ import ctypes as C
 import json
 import math
 import os
+import random
 import time
 
 import numpy as np
@@ -280,14 +281,21 @@ class GPT:
         for i in range(max_new_tokens):
             idx_cond = history[-n_ctx:]
             startTime = time.perf_counter()
-            logits = self.run(idx_cond)
+            h = self._history
+            cached = len(h) > 0 and len(idx_cond) == len(h) + 1 and len(idx_cond) <= n_ctx and idx_cond[:-1] == h
+            if cached and 1 <= top_k <= 1024 and temperature > 0:
+                # the window extends the cached one by a token: that token goes in, the next one is
+                # selected on the device with this draw, and the logits are never read back
+                idx_next = int(self.decode_sample(idx_cond[-1], 1, top_k, temperature, [random.random()])[0])
+            else:
+                logits = self.run(idx_cond)
+                sel = sampling.selectTopK(logits, top_k) if top_k != 1 else \
+                    {"topKIndices": [int(np.argmax(logits))], "topKProbs": [float(np.max(logits))]}
+                probs = sampling.cpuSoftmax(sel["topKProbs"], temperature)
+                idx_next = sel["topKIndices"][sampling.sampleFromDistribution(probs)]
             lapsed = (time.perf_counter() - startTime) * 1000.0
             if i >= warmupRuns:
                 totalTime += lapsed
-            sel = sampling.selectTopK(logits, top_k) if top_k != 1 else \
-                {"topKIndices": [int(np.argmax(logits))], "topKProbs": [float(np.max(logits))]}
-            probs = sampling.cpuSoftmax(sel["topKProbs"], temperature)
-            idx_next = sel["topKIndices"][sampling.sampleFromDistribution(probs)]
             history = history + [idx_next]
             yield self.tokenizer.decode([idx_next]) if self.tokenizer else idx_next
         self.averageMs = totalTime / max(1, max_new_tokens - warmupRuns)
