@@ -132,3 +132,24 @@ def test_decode_sample_follows_the_reference_loop(device, mode, top_k):
 def _lib_error():
     from webgpt_amd import _lib
     return _lib.WgptError
+
+
+@pytest.mark.gpu
+def test_decode_sample_rejects_bad_arguments(device):
+    from webgpt_amd import _lib
+    from webgpt_amd.model import GPT
+    cfg = small_cfg(n_ctx=8)
+    gpt = GPT(None, "char", tensors=make_model(cfg, 1), params=synth.model_params(cfg))
+    gpt.initialize()
+    try:
+        gpt.prefill([1, 2, 3])
+        for args, msg in (((4, 1, 0, 1.0, [0.5]), "top_k"), ((4, 1, 2000, 1.0, [0.5]), "top_k"), ((4, 1, 2, 0.0, [0.5]), "temperature"),
+                          ((4, 1, 2, 1.0, [1.0]), r"u\[0\]"), ((cfg["vocab_size"], 1, 2, 1.0, [0.5]), "outside"),
+                          ((4, 6, 2, 1.0, [0.5] * 6), "exceed")):
+            with pytest.raises(_lib.WgptError, match=msg):
+                gpt.decode_sample(*args)
+        with pytest.raises(ValueError, match="one uniform draw per step"):
+            gpt.decode_sample(4, 2, 2, 1.0, [0.5])
+        assert len(gpt.decode_sample(4, 2, 3, 1.0, [0.1, 0.9])) == 2     # still usable afterwards
+    finally:
+        gpt.unloadBuffers()
