@@ -141,7 +141,7 @@ def test_attention_values_known_answer(device):
     assert np.allclose(got, np.tile(vrow, (T, 1)), rtol=1e-6)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8, 4), (1, 1600, 1600), (1, 4800, 1600), (1, 1600, 6400), (3, 264, 100), (40, 136, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 4), (1, 1600, 1600), (1, 4800, 1600), (1, 1600, 6400), (3, 264, 100), (40, 136, 64), (130, 264, 100), (300, 4800, 1600), (512, 1600, 6400)])
 def test_int8_matmul_and_bit_exact_dequant(device, M, N, K):
     A = rnd(M, K)
     q = RNG.integers(-127, 128, (K, N))

@@ -118,8 +118,14 @@ int wgpt_matmul_bias_i8(int M, int N, int K, wgpt_buf A, wgpt_buf Wq, wgpt_buf s
     int rc = scratch(0, sizeof(float) * gemv_workspace_floats(M, N, K), &ws);
     if (rc) return rc;
     e = launch_gemv_kn_i8(M, N, K, a, K, wq, N / 4, sc, b, c, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
+  } else if (M >= 16) {
+    // Dense contraction on the matrix cores, words dequantised on their way into LDS (same arithmetic).
+    void* ws;
+    int rc = scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
+    if (rc) return rc;
+    e = launch_gemm_i8(M, N, K, a, K, wq, N / 4, sc, b, c, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   } else {
-    // Dense contraction: dequantise once (same arithmetic), then the fp32 GEMM.
+    // A few rows more than the matrix-vector kernel takes: dequantise once (same arithmetic), then the fp32 tile kernel.
     void* wf;
     int rc = scratch(1, sizeof(float) * (size_t)K * N, &wf);
     if (rc) return rc;

@@ -28,6 +28,10 @@ hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const fl
 size_t gemm_workspace_floats(int M, int N);
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
                        float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
+// Same with the packed int8 weights of other/int8-gemm.js (Wq[K, ldwq] words, scale[N]), dequantised inside
+// the kernel; M >= 16.
+hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
+                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
 
 // int8 weight-only variants: Wq is [K, ldwq] words holding 4 columns each.
 hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,

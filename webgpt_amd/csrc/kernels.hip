@@ -278,10 +278,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // With kchunk < K (split-K) slice blockIdx.z covers k in [z*kchunk, (z+1)*kchunk) and
 // writes its raw partial sums to C + z*M*ldc (bias, epilogue: gemv_reduce afterwards).
-template <int TM, int TN, int BK>
+// I8W: W is the packed int8 matrix of other/int8-gemm.js:36-43 (`Wv` points to [K, ldw] words of four
+// consecutive columns, `wscale` to the per-column scales); a thread's word of a step is
+// dequantised on its way into LDS with the arithmetic of unpackInt8x4, so the matrix cores
+// see exactly the weights wgpt_dequant_i8 would write, without the trip through memory.
+template <int TM, int TN, int BK, bool I8W>
 __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
-                                                 const float* __restrict__ W, int ldw, const float* __restrict__ bias,
-                                                 float* C, int ldc, int epi, const float* resid) {
+                                                 const void* __restrict__ Wv, int ldw, const float* __restrict__ wscale,
+                                                 const float* __restrict__ bias, float* C, int ldc, int epi, const float* resid) {
+  const float* W = static_cast<const float*>(Wv);
+  const int32_t* Wq = static_cast<const int32_t*>(Wv);
   constexpr int AST = BK + 4;                // floats per staged A row (16-byte aligned, odd multiple of 4 banks)
   constexpr int RB = TM / 64, CB = TN / 64;  // 32x32 accumulator blocks per wave
   constexpr int KQ = BK / 4;                 // float4 per A row of a step
@@ -297,7 +303,10 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
   const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
   const int arow = tid / KQ, akq = (tid % KQ) * 4;
   const int brow = tid / (TN / 4), bnq = (tid % (TN / 4)) * 4;
-  float4 ga[NA], gb[NB];
+  float4 ga[NA], gb[I8W ? 1 : NB];
+  int32_t gq[I8W ? NB : 1];  // packed words of the step, unpacked when they are staged
+  float4 sc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (I8W && n0 + bnq < N) sc4 = ld4(wscale + n0 + bnq);
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int r = 0; r < NA; ++r) {
@@ -307,7 +316,8 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
       const int k = k0 + brow + r * BROWS;
-      gb[r] = (k < K && n0 + bnq < N) ? ld4(W + (size_t)k * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (I8W) gq[I8W ? r : 0] = (k < K && n0 + bnq < N) ? Wq[(size_t)k * ldw + ((n0 + bnq) >> 2)] : 0;
+      else gb[I8W ? 0 : r] = (k < K && n0 + bnq < N) ? ld4(W + (size_t)k * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
   auto stage = [&](int st) {
@@ -319,7 +329,8 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
       *reinterpret_cast<float2*>(d + HK) = make_float2(ga[r].y, ga[r].w);
     }
 #pragma unroll
-    for (int r = 0; r < NB; ++r) st4(Bs[st] + (brow + r * BROWS) * TN + bnq, gb[r]);
+    for (int r = 0; r < NB; ++r)
+      st4(Bs[st] + (brow + r * BROWS) * TN + bnq, I8W ? unpack_i8x4(gq[I8W ? r : 0], sc4) : gb[I8W ? 0 : r]);
   };
   f32x16 acc[RB][CB];
 #pragma unroll
@@ -1061,18 +1072,33 @@ hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const fl
 size_t gemm_workspace_floats(int M, int N) { return (size_t)8 * M * N; }
 
 namespace {
-template <int TM, int TN, int BK>
-void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const float* W, int ldw, const float* bias, float* C,
-                   int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+template <int TM, int TN, int BK, bool I8W>
+void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const void* W, int ldw, const float* wscale,
+                   const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
   const dim3 grid(cdiv(N, TN), cdiv(M, TM), S);
   if (S == 1) {
-    gemm_mfma<TM, TN, BK><<<grid, WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+    gemm_mfma<TM, TN, BK, I8W><<<grid, WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid);
   } else {
     // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
     const int kchunk = (int)cdiv(cdiv(K, S), BK) * BK;
-    gemm_mfma<TM, TN, BK><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
+    gemm_mfma<TM, TN, BK, I8W><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, nullptr, workspace, N, EPI_NONE, nullptr);
     gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
   }
+}
+
+// 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
+// best or within 3 % of it from 128 to 1024 rows); then split K (at most 8 ways, slices of
+// at least 128) until there are two workgroups per compute unit.
+template <bool I8W>
+void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int ldw, const float* wscale, const float* bias,
+              float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  const bool big = (size_t)cdiv(M, 128) * cdiv(N, 128) >= 512;
+  const int t = big ? 128 : 64;
+  int S = 1;
+  const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
+  while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
+  if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, s);
+  else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, s);
 }
 }  // namespace
 
@@ -1083,16 +1109,14 @@ hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float
     gemm_tile64<<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
     return hipGetLastError();
   }
-  // 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
-  // best or within 3 % of it from 128 to 1024 rows); then split K (at most 8 ways, slices of
-  // at least 128) until there are two workgroups per compute unit.
-  const bool big = (size_t)cdiv(M, 128) * cdiv(N, 128) >= 512;
-  const int t = big ? 128 : 64;
-  int S = 1;
-  const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
-  while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
-  if (big) run_gemm_mfma<128, 128, 32>(M, N, K, S, A, lda, W, ldw, bias, C, ldc, epi, resid, workspace, s);
-  else run_gemm_mfma<64, 64, 32>(M, N, K, S, A, lda, W, ldw, bias, C, ldc, epi, resid, workspace, s);
+  run_gemm<false>(M, N, K, A, lda, W, ldw, nullptr, bias, C, ldc, epi, resid, workspace, s);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
+                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  if (M < 16 || (N & 3)) return hipErrorInvalidValue;
+  run_gemm<true>(M, N, K, A, lda, Wq, ldwq, scale, bias, C, ldc, epi, resid, workspace, s);
   return hipGetLastError();
 }
 

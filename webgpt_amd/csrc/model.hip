@@ -95,6 +95,8 @@ static int linear(Model* m, int M, int N, int K, const float* A, int lda, const 
   if (w.q) {
     if (M <= GEMV_MAX_ROWS) {
       e = launch_gemv_kn_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
+    } else if (M >= 16) {
+      e = launch_gemm_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
     } else {
       e = launch_dequant_i8(K, N, w.q, N / 4, w.s, m->dq, N, s);
       if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s);
