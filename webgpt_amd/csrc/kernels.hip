@@ -265,11 +265,13 @@ __global__ __launch_bounds__(WG) void gemm_tile64(int M, int N, int K, const flo
 // (16 VGPRs per lane). Workgroup tile TM x TN (64 or 128 each), four waves in a 2x2
 // arrangement, each owning (TM/2) x (TN/2) of C as RB x CB accumulator blocks, so an
 // operand fragment read from LDS feeds CB (or RB) instructions. K advances in steps
-// of BK = 32 through two LDS stages: the next step's global loads are in flight while
-// the current one is multiplied and land in the other stage (one barrier per step).
+// of BK = 32 through two LDS stages (one barrier per step); inside a step every wave
+// interleaves its matrix instructions with the LDS reads of the next quarter-step, the
+// global loads of a later step and the move of the next step into the other stage.
 // A is staged as [m][BK + 4] with the k of a step permuted to (k odd, k / 2), so the
 // values a lane feeds to four consecutive instructions are one 128-bit read; W as
-// [k][n].
+// [k][n], odd k with the two 32-column halves of a row swapped so that the two half-waves
+// of an operand read (k and k + 1) use different LDS banks.
 // Operand lane mapping of the instruction: lane l supplies A[row l%32][k l/32] and
 // W[k l/32][col l%32]; accumulator register r of lane l is
 // C[row (r/4)*8 + (l/32)*4 + r%4][col l%32].
@@ -296,41 +298,66 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
   constexpr int BROWS = WG / (TN / 4);       // W rows covered by one pass of the workgroup
   constexpr int NB = BK / BROWS;             // float4 per thread of the W tile of a step
   constexpr int HK = BK / 2;                 // MFMA instructions per step and accumulator block
+  constexpr int NQ = HK / 4;                 // quarters of a step: four k pairs each
+  constexpr int BST = TN;                    // floats per staged W row (odd rows swap their 32-column halves)
   __shared__ __attribute__((aligned(16))) float As[2][TM * AST];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BK * TN];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * BST];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
   const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
   const int arow = tid / KQ, akq = (tid % KQ) * 4;
   const int brow = tid / (TN / 4), bnq = (tid % (TN / 4)) * 4;
-  float4 ga[NA], gb[I8W ? 1 : NB];
-  int32_t gq[I8W ? NB : 1];  // packed words of the step, unpacked when they are staged
+  // D register sets of global data: a step's tile is fetched D steps ahead of its use and moves into
+  // LDS one step ahead; with two sets, set p holds the steps of parity p
+  constexpr int D = RB * CB == 1 ? 2 : 1;  // the large tile has registers for one set only
+  float4 ga[D][NA], gb[D][I8W ? 1 : NB];
+  int32_t gq[D][I8W ? NB : 1];  // packed words of the step, unpacked when they are staged
   float4 sc4 = make_float4(0.f, 0.f, 0.f, 0.f);
   if (I8W && n0 + bnq < N) sc4 = ld4(wscale + n0 + bnq);
-  auto fetch = [&](int k0) {
+  // Every global load is unconditional and in bounds: rows beyond M and columns beyond N repeat the
+  // last valid ones (their results are never stored), k beyond the slice repeats its last values and is
+  // zeroed when the step is staged. (A load under a bounds branch makes the compiler wait for it on
+  // the spot, which exposes the whole memory latency in every step.)
+  const float* arp[NA];
 #pragma unroll
-    for (int r = 0; r < NA; ++r) {
-      const int m = m0 + arow + r * AROWS;
-      ga[r] = (m < M && k0 + akq < K) ? ld4(A + (size_t)m * lda + k0 + akq) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+  for (int r = 0; r < NA; ++r) {
+    const int m = m0 + arow + r * AROWS;
+    arp[r] = A + (size_t)(m < M ? m : M - 1) * lda;
+  }
+  const int ncl = n0 + bnq < N ? n0 + bnq : N - 4;
+  int kf[D] = {};  // first k of the step held by each set
+  auto fetch = [&](auto P, int k0) {
+    constexpr int p = decltype(P)::value;
+    kf[p] = k0;
+    const int ka = k0 + akq < K ? k0 + akq : K - 4;
+#pragma unroll
+    for (int r = 0; r < NA; ++r) ga[p][r] = ld4(arp[r] + ka);
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
       const int k = k0 + brow + r * BROWS;
-      if (I8W) gq[I8W ? r : 0] = (k < K && n0 + bnq < N) ? Wq[(size_t)k * ldw + ((n0 + bnq) >> 2)] : 0;
-      else gb[I8W ? 0 : r] = (k < K && n0 + bnq < N) ? ld4(W + (size_t)k * ldw + n0 + bnq) : make_float4(0.f, 0.f, 0.f, 0.f);
+      const size_t kc = (size_t)(k < K ? k : K - 1);
+      if (I8W) gq[p][I8W ? r : 0] = Wq[kc * ldw + (ncl >> 2)];
+      else gb[p][I8W ? 0 : r] = ld4(W + kc * ldw + ncl);
     }
   };
-  auto stage = [&](int st) {
+  auto stage = [&](auto P, int st) {
+    constexpr int p = decltype(P)::value;
+    const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool ain = kf[p] + akq < K;
 #pragma unroll
     for (int r = 0; r < NA; ++r) {
       // k = akq + j goes to slot (k & 1) * HK + k / 2: (x, z) are the even k, (y, w) the odd
+      const float4 v = ain ? ga[p][r] : z;
       float* d = As[st] + (arow + r * AROWS) * AST + (akq >> 1);
-      *reinterpret_cast<float2*>(d) = make_float2(ga[r].x, ga[r].z);
-      *reinterpret_cast<float2*>(d + HK) = make_float2(ga[r].y, ga[r].w);
+      *reinterpret_cast<float2*>(d) = make_float2(v.x, v.z);
+      *reinterpret_cast<float2*>(d + HK) = make_float2(v.y, v.w);
     }
 #pragma unroll
-    for (int r = 0; r < NB; ++r)
-      st4(Bs[st] + (brow + r * BROWS) * TN + bnq, I8W ? unpack_i8x4(gq[I8W ? r : 0], sc4) : gb[I8W ? 0 : r]);
+    for (int r = 0; r < NB; ++r) {
+      const bool bin = kf[p] + brow + r * BROWS < K;
+      const float4 v = I8W ? unpack_i8x4(gq[p][I8W ? r : 0], sc4) : gb[p][I8W ? 0 : r];
+      st4(Bs[st] + (brow + r * BROWS) * BST + (bnq ^ (((brow + r * BROWS) & 1) << 5)), bin ? v : z);
+    }
   };
   f32x16 acc[RB][CB];
 #pragma unroll
@@ -340,54 +367,108 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[r][c][i] = 0.f;
 
+  const int h = lane >> 5, l32 = lane & 31;
+  // operands of quarter q of the step in LDS stage st: four k pairs per accumulator row / column block
+  auto operands = [&](float (&av)[RB][4], float (&bv)[CB][4], int st, int q) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + q * 4);
+      av[r][0] = v.x; av[r][1] = v.y; av[r][2] = v.z; av[r][3] = v.w;
+    }
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      const float* bp = Bs[st] + (h + 8 * q) * BST + ((wn + c * 32 + l32) ^ (h << 5));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bv[c][i] = bp[2 * i * BST];
+    }
+  };
+  auto multiply = [&](const float (&av)[RB][4], const float (&bv)[CB][4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int c = 0; c < CB; ++c) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[r][i], bv[c][i], acc[r][c], 0, 0, 0);
+  };
+
+  // requested before the main loop so that the epilogue does not wait for it
+  float biasv[CB];
+#pragma unroll
+  for (int c = 0; c < CB; ++c) {
+    const int n = n0 + wn + c * 32 + l32;
+    biasv[c] = (bias && n < N) ? bias[n] : 0.f;
+  }
   const int kbeg = blockIdx.z * kchunk;
   const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
   C += (size_t)blockIdx.z * M * ldc;
   K = kend;
-  fetch(kbeg);
-  stage(0);
+  typedef std::integral_constant<int, 0> P0;
+  typedef std::integral_constant<int, 1> P1;
+  fetch(P0(), kbeg);
+  stage(P0(), 0);
+  if constexpr (D == 2) {
+    if (kbeg + BK < kend) fetch(P1(), kbeg + BK);
+  }
   __syncthreads();
+  float av[2][RB][4], bv[2][CB][4];  // operands of the quarter being multiplied and of the next one
+  operands(av[0], bv[0], 0, 0);
   int st = 0;
-  const int h = lane >> 5, l32 = lane & 31;
-  for (int k0 = kbeg; k0 < kend; k0 += BK) {
-    const bool more = k0 + BK < kend;
-    if (more) fetch(k0 + BK);
-    // QS quarter-steps of operands are read from LDS at a time, then their matrix instructions run
-    // back to back: the whole step for the small tile (32 registers), a quarter for the large one
-    constexpr int QS = RB * CB == 1 ? HK / 4 : 1;
-#pragma unroll
-    for (int q0 = 0; q0 < HK / 4; q0 += QS) {
-      float av[RB][4 * QS], bv[CB][4 * QS];
-#pragma unroll
-      for (int q = 0; q < QS; ++q) {
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-          const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + (q0 + q) * 4);
-          av[r][4 * q] = v.x; av[r][4 * q + 1] = v.y; av[r][4 * q + 2] = v.z; av[r][4 * q + 3] = v.w;
-        }
-#pragma unroll
-        for (int c = 0; c < CB; ++c) {
-          const float* bp = Bs[st] + (h + 8 * (q0 + q)) * TN + wn + c * 32 + l32;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) bv[c][4 * q + i] = bp[2 * i * TN];
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4 * QS; ++i)
-#pragma unroll
-        for (int r = 0; r < RB; ++r)
-#pragma unroll
-          for (int c = 0; c < CB; ++c) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[r][i], bv[c][i], acc[r][c], 0, 0, 0);
+  // One K step. A wave keeps its own matrix pipe fed: while the instructions of a quarter run, the
+  // operands of the next quarter are on their way from LDS, the global loads of a later step (D steps
+  // ahead) are in flight, and the next step's tile moves from registers into the other LDS stage. The
+  // last quarter is multiplied after the barrier, behind the request for the next step's first
+  // operands. (Leaving the overlap to a second wave of the SIMD does not work: the workgroups of a
+  // compute unit fall into step with each other and stall together.)
+  // FETCH / STAGE are compile-time so that the steady state is straight-line code: with a branch
+  // around the loads the compiler can no longer tell which of them are outstanding and waits early.
+  auto kstep = [&](auto P, auto FETCH, auto STAGE, int k0) {
+    constexpr int p = decltype(P)::value;
+    static_assert(NQ % 2 == 0, "the last quarter of a step must sit in operand set 1");
+    if (decltype(FETCH)::value) {
+      fetch(std::integral_constant<int, D == 2 ? p : 0>(), k0 + D * BK);  // that set was staged a step ago
+      __builtin_amdgcn_sched_barrier(0);  // keep the loads here, at the head of the step
     }
-    if (more) stage(st ^ 1);
-    __syncthreads();
-    st ^= 1;
+#pragma unroll
+    for (int q = 0; q < NQ - 1; ++q) {
+      operands(av[(q + 1) & 1], bv[(q + 1) & 1], st, q + 1);
+      multiply(av[q & 1], bv[q & 1]);
+    }
+    if (decltype(STAGE)::value) {
+      __builtin_amdgcn_sched_barrier(0);  // nothing of the move into LDS (it waits for the loads) drifts up
+      stage(std::integral_constant<int, D == 2 ? 1 - p : 0>(), st ^ 1);
+      __syncthreads();
+      st ^= 1;
+      operands(av[0], bv[0], st, 0);
+    }
+    multiply(av[1], bv[1]);
+  };
+  const std::true_type yes;
+  const std::false_type no;
+  int k0 = kbeg;
+  if constexpr (D == 2) {
+    for (; k0 + 3 * BK < kend; k0 += 2 * BK) {
+      kstep(P0(), yes, yes, k0);
+      kstep(P1(), yes, yes, k0 + BK);
+    }
+    if (k0 + 2 * BK < kend) {  // three steps left
+      kstep(P0(), yes, yes, k0);
+      kstep(P1(), no, yes, k0 + BK);
+      kstep(P0(), no, no, k0 + 2 * BK);
+    } else if (k0 + BK < kend) {  // two
+      kstep(P0(), no, yes, k0);
+      kstep(P1(), no, no, k0 + BK);
+    } else if (k0 < kend) {  // one
+      kstep(P0(), no, no, k0);
+    }
+  } else {
+    for (; k0 + BK < kend; k0 += BK) kstep(P0(), yes, yes, k0);
+    if (k0 < kend) kstep(P0(), no, no, k0);
   }
 #pragma unroll
   for (int c = 0; c < CB; ++c) {
     const int n = n0 + wn + c * 32 + l32;
     if (n >= N) continue;
-    const float bvs = bias ? bias[n] : 0.f;
+    const float bvs = biasv[c];
 #pragma unroll
     for (int r = 0; r < RB; ++r)
 #pragma unroll
