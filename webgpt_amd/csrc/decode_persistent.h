@@ -13,6 +13,7 @@ constexpr int PD_THREADS = 512;  // threads per workgroup
 constexpr int PD_GRID = 256;     // workgroups: one per compute unit of an MI355X
 constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase
 constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
+constexpr int PD_COLP = 256;     // floats of one workgroup's column parameters of a layer (4 phases x 32 columns x {bias, scale})
 constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
@@ -49,6 +50,7 @@ struct PersistentArgs {
   const void* slabs;
   size_t slab_stride, slab_offC, slab_offD, slab_offE;
   const float* lparams;  // [L][22d] small per-layer parameters (LayerParamOffsets)
+  const float* colparams;  // [L][PD_GRID][PD_COLP] biases and int8 scales / 127 per workgroup (build_colparams)
   const float *wte, *wpe, *lnf_g, *lnf_b;
   float* kv;  // [L][2][H][ctx][hs]
   // {value, epoch} exchange buffers
@@ -82,6 +84,10 @@ hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const 
 hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* beta, const float* bias, float* out, hipStream_t s);
 // Same for int8 words Wq[K, ldwq] (4 columns per word): one word per item lane.
 hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g, int32_t* slab, hipStream_t s);
+// Biases and (int8) column scales / 127 of lparams re-laid per layer and workgroup: float t of a block is
+// parameter kind t / 128 (bias, scale) of local column t % 32 of linear phase (t / 32) % 4, zero where the
+// workgroup has no such column.
+hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype, float* out, hipStream_t s);
 // Model shapes the persistent kernel is instantiated for.
 bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype);
 // Epochs consumed by one decode step.

@@ -202,14 +202,42 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
   }
 }
 
-// Registers of one linear phase: this wave's share of the weight slab (MAXI items per
-// lane) and the bias (int8: also scale / 127) of the column this lane finishes.
+// Registers of one linear phase: this wave's share of the weight slab (MAXI items per lane).
 template <int MAXI, bool I8>
 struct WSet {
   typename std::conditional<I8, int, float4>::type w[MAXI];  // an int8 item is one word per lane
-  float bias;
-  float cscale;
 };
+
+// Per-layer column parameters of a workgroup in LDS: bias of local column c of phase ph at
+// colp[ph * LPW + c], int8 column scale / 127 at colp[(4 + ph) * LPW + c]. They are requested
+// into one register per thread a phase before the layer starts and deposited next to the
+// layer's first input row; build_colparams lays them out per layer and workgroup. (Held in registers of the finishing lanes for the length of a
+// phase they were the first values the compiler spilled, and a spill of a value just
+// requested waits for every load in flight, the weights of the next phase included.)
+constexpr int LPW = PD_COLP / 8;  // columns of a phase per workgroup, at most
+
+// Linear phases of a layer, in execution order.
+enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
+
+// Bias and int8 scale of local column c of phase ph, read ahead of the dot products (any lane may ask:
+// c wraps inside the phase's LPW slots).
+struct ColParams {
+  float bias, scale;
+};
+template <bool I8>
+__device__ __forceinline__ ColParams col_params(const float* colp, int ph, int c) {
+  c &= LPW - 1;
+  ColParams r;
+  r.bias = colp[ph * LPW + c];
+  r.scale = I8 ? colp[(4 + ph) * LPW + c] : 1.f;
+  return r;
+}
+// Finished value of a column from its dot product: the int8 column scale, the bias last.
+template <bool I8>
+__device__ __forceinline__ float finish(float dot, const ColParams& cp) {
+  return (I8 ? dot * cp.scale : dot) + cp.bias;
+}
+
 
 // The four signed bytes of a word as floats (element e in bits 8e..8e+7,
 // other/int8-gemm.js:36-43).
@@ -244,8 +272,7 @@ __device__ __forceinline__ float4 to_float4(int v) { return bytes_to_float4(v); 
 // word of four int8, per lane) of segment seg of local column c. `ncols` is the
 // number of columns this workgroup finishes (CPW except at the ragged end).
 template <class P, class WS, class T>
-__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, const float* __restrict__ bias,
-                                           const float* __restrict__ scale, int ncols, int wg, int wave, int lane) {
+__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, int ncols, int wg, int wave, int lane) {
   const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
   if (P::WHOLE) {
 #pragma unroll
@@ -271,12 +298,6 @@ __device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, c
       }
     });
   }
-  // the lane that finishes a column: lane cc of the wave that holds it (WHOLE), else thread c
-  const int l = opaque(lane);
-  const int c = P::WHOLE ? wave + l * NW : (int)threadIdx.x;
-  const bool mine = (P::WHOLE ? l < P::CW : true) && c < ncols;
-  ws.bias = mine ? bias[wg * P::CPW + c] : 0.f;
-  if (std::is_same<T, int>::value) ws.cscale = mine ? scale[wg * P::CPW + c] / 127.0f : 0.f;
 }
 
 // LayerNorm parameters travel global memory -> registers (requested with the weights
@@ -411,11 +432,12 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
 // Second MLP matrix: either layout. Whole columns leave residual + column in pubE;
 // split columns leave per-wave partials in part (finished after the barrier).
 template <class P, bool I8, class WS>
-__device__ __forceinline__ void phase_e(const WS& ws, const float* xs, float* part, const float* pubC, float* pubE, int ncols,
-                                        bool fin, int fc, int wave, int lane) {
+__device__ __forceinline__ void phase_e(const WS& ws, const float* xs, float* part, const float* pubC, float* pubE,
+                                        const float* colp, int ncols, bool fin, int fc, int wave, int lane) {
   if constexpr (P::WHOLE) {
+    const ColParams cp = col_params<I8>(colp, PH_FC2, fc);
     const float dot = gemv_whole<P, false, false>(ws, xs, nullptr, ncols, wave, lane);
-    if (fin) pubE[fc] = pubC[fc] + ((I8 ? dot * ws.cscale : dot) + ws.bias);
+    if (fin) pubE[fc] = pubC[fc] + finish<I8>(dot, cp);
   } else {
     gemv_split<P>(ws, xs, part, ncols, wave, lane);
   }
@@ -432,11 +454,6 @@ __device__ __forceinline__ float column_sum(const float* part, int c) {
   return s;
 }
 
-// Finished value of a column from its dot product: the int8 column scale, the bias last.
-template <bool I8, class WS>
-__device__ __forceinline__ float finish(float dot, const WS& ws) {
-  return (I8 ? dot * ws.cscale : dot) + ws.bias;
-}
 
 #ifdef WGPT_TRACE
 #define TRACE(slot)                                                                              \
@@ -471,8 +488,6 @@ __device__ __forceinline__ void wave_first(float& v, int& i) {
   }
 }
 
-// Linear phases of a layer, in execution order.
-enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
@@ -521,6 +536,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float* pubC = pubA + PA::CPW;   // [PC::CPW] residual stream after the attention projection
   float* pubD = pubC + PC::CPW;   // [PD::CPW] finished c_fc columns
   float* pubE = pubD + PD::CPW;   // [PE::CPW] residual stream after the MLP (whole-column layout only)
+  float* colp = pubE + PE::CPW;   // [8 * LPW] biases and int8 column scales of this workgroup's columns of the layer
+  static_assert(PA::CPW <= LPW && PC::CPW <= LPW && PD::CPW <= LPW && PE::CPW <= LPW, "a phase has more columns per workgroup than colp holds");
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
@@ -556,7 +573,20 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   unsigned ep = a.ebase;
   int tok = a.tok[0];
 
-  load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+  // the layer's block for this workgroup is already in the layout of colp (build_colparams): one load per thread
+  float preg = 0.f;
+  auto request_params = [&](int layer) {
+    // unconditional (the upper half of the workgroup re-reads the lower half's words): after a load
+    // under a branch the compiler waits for every load in flight where the paths join
+    preg = a.colparams[((size_t)layer * PD_GRID + wg) * PD_COLP + (opaque(tid) & (PD_COLP - 1))];
+  };
+  auto deposit_params = [&]() {
+    const int t = opaque(tid);
+    if (t < PD_COLP) colp[t] = preg;
+  };
+  request_params(0);
+  load_items<PA>(wX, slabs, ncA, wg, wave, lane);
+  deposit_params();
   // FOLD: only the final LayerNorm has parameters, and they stay in lnp for good
   if (FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
   else request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
@@ -566,8 +596,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   for (int step = 0; step < a.nsteps; ++step) {
     const int pos = a.pos0 + step;
     TRACE(0);
+#ifdef WGPT_TRACE
+    if (a.trace && tid == 0 && step == a.nsteps - 1) a.trace[(size_t)wg * 512 + 500] = __builtin_readcyclecounter();
+#endif
     // ---- embedding: every workgroup builds the row itself (instructions.js:795-821) ----
     for (int e = tid; e < D; e += NT) xs0[e] = a.wte[(size_t)tok * D + e] + a.wpe[(size_t)pos * D + e];
+    if (step > 0) deposit_params();  // the first layer's, requested during the last layer of the token before
     __syncthreads();
 
     // slice of positions 0..pos for the attention role
@@ -593,21 +627,23 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (li > 0) {
           poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0], a.spin_limit);
           if (!FOLD) deposit_ln<D>(lnreg, lnp);
+          deposit_params();
           __syncthreads();
           if (sh.bail) return;
         }
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) load_items<PC>(wY, slab + a.slab_offC, lp + po.bC, lp + po.sC, ncC, wg, wave, lane);
+        if (DUAL) load_items<PC>(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
+        const ColParams cp = col_params<I8>(colp, PH, fc);
         const float dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane);
         TRACE5(2);
-        if (finA) pubA[fc] = finish<I8>(dot, wX);
+        if (finA) pubA[fc] = finish<I8>(dot, cp);
         __syncthreads();
         ++ep;
         if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
         TRACE5(4);
-        if (!DUAL) load_items<PC>(wY, slab + a.slab_offC, lp + po.bC, lp + po.sC, ncC, wg, wave, lane);
+        if (!DUAL) load_items<PC>(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -736,7 +772,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         if (DUAL) {
-          load_items<PD>(wX, slab + a.slab_offD, lp + po.bD, lp + po.sD, ncD, wg, wave, lane);
+          load_items<PD>(wX, slab + a.slab_offD, ncD, wg, wave, lane);
           if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         }
         // merge of the slices of each head (flash-decoding): element e of head h is
@@ -770,15 +806,16 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         __syncthreads();
         TRACE5(1);
+        const ColParams cp = col_params<I8>(colp, PH, fc);
         const float dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
         TRACE5(2);
-        if (finC) pubC[fc] = own_r + finish<I8>(dot, wY);  // model.js:159
+        if (finC) pubC[fc] = own_r + finish<I8>(dot, cp);  // model.js:159
         __syncthreads();
         ++ep;
         if (tid < ncC) publish(a.bufR1 + wg * PC::CPW + tid, pubC[tid], ep);
         TRACE5(4);
         if (!DUAL) {
-          load_items<PD>(wX, slab + a.slab_offD, lp + po.bD, lp + po.sD, ncD, wg, wave, lane);
+          load_items<PD>(wX, slab + a.slab_offD, ncD, wg, wave, lane);
           if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         }
         TRACE5(5);
@@ -792,15 +829,16 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
+        if (DUAL) load_items<PE>(wY, slab + a.slab_offE, ncE, wg, wave, lane);
+        const ColParams cp = col_params<I8>(colp, PH, fc);
         const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane);
         TRACE5(2);
-        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, wX));  // model.js:188
+        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
         ++ep;
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
         TRACE5(4);
-        if (!DUAL) load_items<PE>(wY, slab + a.slab_offE, lp + po.bE, lp + po.sE, ncE, wg, wave, lane);
+        if (!DUAL) load_items<PE>(wY, slab + a.slab_offE, ncE, wg, wave, lane);
         TRACE5(5);
       }
 
@@ -812,11 +850,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // sets, already the first layer's share for the next token)
         auto request_next = [&]() {
           if (li + 1 < a.L) {
-            load_items<PA>(wX, slab + a.slab_stride, lp + po.stride + po.bA, lp + po.stride + po.sA, ncA, wg, wave, lane);
+            load_items<PA>(wX, slab + a.slab_stride, ncA, wg, wave, lane);
+            request_params(li + 1);
             if (!FOLD) request_ln<D>(lnreg, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
           } else {
             if (!FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
-            if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+            if (step + 1 < a.nsteps) request_params(0);
+            if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, ncA, wg, wave, lane);
           }
         };
         poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
@@ -824,12 +864,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         if (DUAL) request_next();
-        phase_e<PE, I8>(wY, xs1, part, pubC, pubE, ncE, finE, fc, wave, lane);
+        const ColParams cpe = col_params<I8>(colp, PH, tid);  // split columns: thread c finishes local column c
+        phase_e<PE, I8>(wY, xs1, part, pubC, pubE, colp, ncE, finE, fc, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
         if (tid < ncE) {  // model.js:205
-          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(column_sum<PE>(part, tid), wY);
+          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(column_sum<PE>(part, tid), cpe);
           publish(a.bufR2 + wg * PE::CPW + tid, r2, ep);
         }
         TRACE5(4);
@@ -971,8 +1012,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       }
     }
     TRACE(2 + a.L * 8);
+#ifdef WGPT_TRACE
+    if (a.trace && tid == 0 && step == a.nsteps - 1) a.trace[(size_t)wg * 512 + 501] = __builtin_readcyclecounter();
+#endif
     if (step + 1 < a.nsteps) {
-      if (!DUAL) load_items<PA>(wX, slabs, a.lparams + po.bA, a.lparams + po.sA, ncA, wg, wave, lane);
+      if (!DUAL) load_items<PA>(wX, slabs, ncA, wg, wave, lane);
       if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
@@ -1126,13 +1170,33 @@ __global__ void build_slab_i8_kernel(const int32_t* __restrict__ Wq, int ldwq, i
   slab[idx] = (int32_t)out;
 }
 
+// One thread per float of the per-workgroup parameter blocks: out[(layer * G + wg) * PD_COLP + t].
+__global__ void build_colparams_kernel(const float* __restrict__ lparams, int L, int d, int i8, PhaseGeom gA, PhaseGeom gC,
+                                       PhaseGeom gD, PhaseGeom gE, float* __restrict__ out) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)L * PD_GRID * PD_COLP) return;
+  const int t = (int)(idx % PD_COLP), wg = (int)((idx / PD_COLP) % PD_GRID), layer = (int)(idx / ((size_t)PD_COLP * PD_GRID));
+  const int kind = t / (4 * LPW), ph = (t / LPW) & 3, c = t % LPW;
+  const LayerParamOffsets po = layer_param_offsets(d);
+  const PhaseGeom g = ph == PH_QKV ? gA : ph == PH_PROJ ? gC : ph == PH_FC ? gD : gE;
+  const int off = ph == PH_QKV ? (kind ? po.sA : po.bA) : ph == PH_PROJ ? (kind ? po.sC : po.bC)
+                : ph == PH_FC ? (kind ? po.sD : po.bD) : (kind ? po.sE : po.bE);
+  const int col = wg * g.cpw + c;
+  float v = 0.f;
+  if (c < g.cpw && col < g.N && (kind == 0 || i8)) {
+    v = lparams[(size_t)layer * po.stride + off + col];
+    if (kind) v = v / 127.0f;  // other/int8-gemm.js:126-132 divides by 127 before the column scale is applied
+  }
+  out[idx] = v;
+}
+
 template <class C>
 size_t lds_bytes_of() {
   typedef Phases<C> PS;
   constexpr int XS = (C::SD + C::SH) * SEG;
   constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;
   constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
-  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + 16);
+  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + PD_COLP + 16);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
   const size_t one_per_cu = 84 * 1024;
   return need > one_per_cu ? need : one_per_cu;
@@ -1190,6 +1254,13 @@ bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
   if (weight_dtype == 1) return d == 1600 && n_head == 25;
   return (d == 384 && n_head == 6) || (d == 768 && n_head == 12) || (d == 1024 && n_head == 16) ||
          (d == 1280 && n_head == 20);
+}
+
+hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype, float* out, hipStream_t s) {
+  const size_t n = (size_t)L * PD_GRID * PD_COLP;
+  build_colparams_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(lparams, L, d, weight_dtype, make_geom(3 * d, d), make_geom(d, d),
+                                                                      make_geom(4 * d, d), make_geom(d, 4 * d), out);
+  return hipGetLastError();
 }
 
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {

@@ -243,9 +243,13 @@ static int setup_persistent(Model* m) {
       LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_b, l.fc_b, lp + po.bD, rt().stream));
     }
   }
+  float* colparams;
+  if ((rc = dev_alloc(m, sizeof(float) * (size_t)m->L * PD_GRID * PD_COLP, (void**)&colparams))) return rc;
+  LAUNCH(build_colparams(lparams, m->L, d, i8 ? 1 : 0, colparams, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   a.slabs = slabs;
   a.lparams = lparams;
+  a.colparams = colparams;
   a.wte = m->wte; a.wpe = m->wpe; a.lnf_g = m->lnf_g; a.lnf_b = m->lnf_b;
   a.kv = m->kv;
   const size_t words = (size_t)3 * d + attw + d + hid + d + 2 * PD_TOPK * G;
