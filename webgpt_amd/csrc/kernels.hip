@@ -284,7 +284,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // consecutive columns, `wscale` to the per-column scales); a thread's word of a step is
 // dequantised on its way into LDS with the arithmetic of unpackInt8x4, so the matrix cores
 // see exactly the weights wgpt_dequant_i8 would write, without the trip through memory.
-template <int TM, int TN, int BK, bool I8W>
+template <int TM, int TN, int BK, bool I8W, bool EXACT>
 __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
                                                  const void* __restrict__ Wv, int ldw, const float* __restrict__ wscale,
                                                  const float* __restrict__ bias, float* C, int ldc, int epi, const float* resid) {
@@ -317,46 +317,66 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
   // Every global load is unconditional and in bounds: rows beyond M and columns beyond N repeat the
   // last valid ones (their results are never stored), k beyond the slice repeats its last values and is
   // zeroed when the step is staged. (A load under a bounds branch makes the compiler wait for it on
-  // the spot, which exposes the whole memory latency in every step.)
-  const float* arp[NA];
+  // the spot, which exposes the whole memory latency in every step.) EXACT: every K slice is whole
+  // steps, so there is nothing to clamp or zero along k, and a step's addresses are a uniform base
+  // plus per-thread offsets: vector-ALU instructions of a step queue behind the matrix instructions
+  // of the other waves of the SIMD, so the fewer the better.
+  const int kbeg = blockIdx.z * kchunk;
+  const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
+  C += (size_t)blockIdx.z * M * ldc;
+  K = kend;
+  const int ncl = n0 + bnq < N ? n0 + bnq : N - 4;
+  unsigned aoff[NA], boff[NB];  // element offsets from the step's first k (A) / first row (W)
 #pragma unroll
   for (int r = 0; r < NA; ++r) {
     const int m = m0 + arow + r * AROWS;
-    arp[r] = A + (size_t)(m < M ? m : M - 1) * lda;
+    aoff[r] = (unsigned)((size_t)(m < M ? m : M - 1) * lda + akq);
   }
-  const int ncl = n0 + bnq < N ? n0 + bnq : N - 4;
+#pragma unroll
+  for (int r = 0; r < NB; ++r) boff[r] = (unsigned)((size_t)(brow + r * BROWS) * ldw + (I8W ? ncl >> 2 : ncl));
   int kf[D] = {};  // first k of the step held by each set
   auto fetch = [&](auto P, int k0) {
     constexpr int p = decltype(P)::value;
     kf[p] = k0;
-    const int ka = k0 + akq < K ? k0 + akq : K - 4;
+    if (EXACT) {
+      const float* at = A + k0;
+      const size_t wrow = (size_t)k0 * ldw;
 #pragma unroll
-    for (int r = 0; r < NA; ++r) ga[p][r] = ld4(arp[r] + ka);
+      for (int r = 0; r < NA; ++r) ga[p][r] = ld4(at + aoff[r]);
 #pragma unroll
-    for (int r = 0; r < NB; ++r) {
-      const int k = k0 + brow + r * BROWS;
-      const size_t kc = (size_t)(k < K ? k : K - 1);
-      if (I8W) gq[p][I8W ? r : 0] = Wq[kc * ldw + (ncl >> 2)];
-      else gb[p][I8W ? 0 : r] = ld4(W + kc * ldw + ncl);
+      for (int r = 0; r < NB; ++r) {
+        if (I8W) gq[p][I8W ? r : 0] = (Wq + wrow)[boff[r]];
+        else gb[p][I8W ? 0 : r] = ld4(W + wrow + boff[r]);
+      }
+    } else {
+      const int ka = k0 + akq < K ? k0 : K - 4 - akq;
+#pragma unroll
+      for (int r = 0; r < NA; ++r) ga[p][r] = ld4(A + ka + aoff[r]);
+#pragma unroll
+      for (int r = 0; r < NB; ++r) {
+        const int k = k0 + brow + r * BROWS;
+        const size_t wrow = (size_t)(k < K ? k0 : K - 1 - brow - r * BROWS) * ldw;
+        if (I8W) gq[p][I8W ? r : 0] = (Wq + wrow)[boff[r]];
+        else gb[p][I8W ? 0 : r] = ld4(W + wrow + boff[r]);
+      }
     }
   };
+  // LDS layouts: A tile as [m][BK + 4], W tile as [k][TN] with the two 32-column halves of every 64 columns
+  // swapped in rows with bit 2 set. Matrix instruction i of quarter q takes k = 8q + 4h + i from half-wave h, so
+  // a lane's four A values of a quarter are one 128-bit read of the unpermuted row, and the two half-waves of
+  // a W read (rows 8q + i and 8q + 4 + i) use different banks.
   auto stage = [&](auto P, int st) {
     constexpr int p = decltype(P)::value;
     const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-    const bool ain = kf[p] + akq < K;
+    const bool ain = EXACT || kf[p] + akq < K;
 #pragma unroll
-    for (int r = 0; r < NA; ++r) {
-      // k = akq + j goes to slot (k & 1) * HK + k / 2: (x, z) are the even k, (y, w) the odd
-      const float4 v = ain ? ga[p][r] : z;
-      float* d = As[st] + (arow + r * AROWS) * AST + (akq >> 1);
-      *reinterpret_cast<float2*>(d) = make_float2(v.x, v.z);
-      *reinterpret_cast<float2*>(d + HK) = make_float2(v.y, v.w);
-    }
+    for (int r = 0; r < NA; ++r) st4(As[st] + (arow + r * AROWS) * AST + akq, ain ? ga[p][r] : z);
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
-      const bool bin = kf[p] + brow + r * BROWS < K;
+      const int row = brow + r * BROWS;
+      const bool bin = EXACT || kf[p] + row < K;
       const float4 v = I8W ? unpack_i8x4(gq[p][I8W ? r : 0], sc4) : gb[p][I8W ? 0 : r];
-      st4(Bs[st] + (brow + r * BROWS) * BST + (bnq ^ (((brow + r * BROWS) & 1) << 5)), bin ? v : z);
+      st4(Bs[st] + row * BST + (bnq ^ (((row >> 2) & 1) << 5)), bin ? v : z);
     }
   };
   f32x16 acc[RB][CB];
@@ -372,14 +392,14 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
   auto operands = [&](float (&av)[RB][4], float (&bv)[CB][4], int st, int q) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + h * HK + q * 4);
+      const float4 v = ld4(As[st] + (wm + r * 32 + l32) * AST + 8 * q + 4 * h);
       av[r][0] = v.x; av[r][1] = v.y; av[r][2] = v.z; av[r][3] = v.w;
     }
 #pragma unroll
     for (int c = 0; c < CB; ++c) {
-      const float* bp = Bs[st] + (h + 8 * q) * BST + ((wn + c * 32 + l32) ^ (h << 5));
+      const float* bp = Bs[st] + (8 * q + 4 * h) * BST + ((wn + c * 32 + l32) ^ (h << 5));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) bv[c][i] = bp[2 * i * BST];
+      for (int i = 0; i < 4; ++i) bv[c][i] = bp[i * BST];
     }
   };
   auto multiply = [&](const float (&av)[RB][4], const float (&bv)[CB][4]) {
@@ -398,10 +418,6 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
     const int n = n0 + wn + c * 32 + l32;
     biasv[c] = (bias && n < N) ? bias[n] : 0.f;
   }
-  const int kbeg = blockIdx.z * kchunk;
-  const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
-  C += (size_t)blockIdx.z * M * ldc;
-  K = kend;
   typedef std::integral_constant<int, 0> P0;
   typedef std::integral_constant<int, 1> P1;
   fetch(P0(), kbeg);
@@ -481,6 +497,194 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
           C[(size_t)m * ldc + n] = v;
         }
       }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The same contraction for problems that give every compute unit one 64 x 128 tile: 512 threads, two
+// groups of four waves (one wave of each group per SIMD); group g owns columns [64g, 64g + 64) of the
+// tile, its waves a 32 x 32 block each. The groups alternate: while one issues the 16 matrix
+// instructions of a K step from registers, the other does its memory work (operands of its next
+// step from LDS into registers, its share of a later tile from registers into LDS, global loads two
+// steps ahead of that), then they swap at a barrier. A SIMD's matrix pipe therefore always has
+// exactly one wave feeding it, and no wave waits for memory between matrix instructions. (With
+// independent workgroups the waves of a SIMD run in step, want the pipe at the same time and stall
+// at the same time.) Tiles of K steps 0, 1, ... alternate between two LDS stages; group 0 multiplies
+// step k in the first half of iteration k, group 1 in the second half. Every load and LDS write is
+// unconditional: tiles beyond the K range are fetched from clamped addresses and staged as zeros.
+// ---------------------------------------------------------------------------
+constexpr int PP_THREADS = 512;
+#ifndef PP_BK
+#define PP_BK 32
+#endif
+constexpr size_t PP_LDS = sizeof(float) * 2 * (64 * (PP_BK + 4) + PP_BK * 128);
+template <int BK>
+__global__ __launch_bounds__(PP_THREADS) void gemm_pingpong(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
+                                                            const float* __restrict__ W, int ldw, const float* __restrict__ bias,
+                                                            float* C, int ldc, int epi, const float* resid) {
+  constexpr int TM = 64, TN = 128, AST = BK + 4, HK = BK / 2;
+  constexpr int NA = BK / 32, NB = BK / 16;  // float4 of A and of W per thread and tile
+  extern __shared__ __attribute__((aligned(16))) float pp_lds[];
+  float* const As = pp_lds;                  // [2][TM * AST]
+  float* const Bs = pp_lds + 2 * TM * AST;   // [2][BK * TN]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = wave >> 2, wq = wave & 3, t = tid & 255;
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  const int wm = (wq >> 1) * 32, wn = g * 64 + (wq & 1) * 32;
+  const int h = lane >> 5, l32 = lane & 31;
+  // this thread's share of a tile: NA float4 of A (row 32g + t / 8, float4 t % 8 + 8j of the row), NB of W (the
+  // group's own columns, rows t / 16 + 16r). Rows beyond M and columns beyond N repeat the last valid ones
+  // (their results are never stored).
+  const int arow = g * 32 + (t >> 3), akq = (t & 7) * 4;
+  const int brow = t >> 4, bnq = g * 64 + (t & 15) * 4;
+  const int ncl = n0 + bnq < N ? n0 + bnq : N - 4;
+  // byte offsets of the thread inside a tile; the tile's own address is uniform and advances with the step,
+  // so that a memory phase issues almost no vector-ALU instructions: those queue behind the other group's
+  // matrix instructions on the same SIMD, LDS and global-memory instructions do not
+  unsigned aoff[NA], boff[NB];
+#pragma unroll
+  for (int j = 0; j < NA; ++j) aoff[j] = (unsigned)(((size_t)(m0 + arow < M ? m0 + arow : M - 1) * lda + akq + 32 * j) * sizeof(float));
+#pragma unroll
+  for (int j = 0; j < NB; ++j) boff[j] = (unsigned)(((size_t)(brow + 16 * j) * ldw + ncl) * sizeof(float));
+
+  const int kbeg = blockIdx.z * kchunk;
+  const int kend = kbeg + kchunk < K ? kbeg + kchunk : K;
+  C += (size_t)blockIdx.z * M * ldc;
+  const int nsteps = (kend - kbeg) / BK;  // the launcher guarantees whole steps
+  const char* Abase = reinterpret_cast<const char*>(A + kbeg);
+  const char* Wbase = reinterpret_cast<const char*>(W + (size_t)kbeg * ldw);
+  const size_t wstep = (size_t)BK * ldw * sizeof(float);
+
+  struct Share {
+    float4 a[NA], b[NB];
+  };
+  auto load_share = [&](int tile) {  // this thread's share of tile `tile` (tiles past the end repeat the last one)
+    const int tc = tile < nsteps ? tile : nsteps - 1;
+    // the tile addresses are uniform: keep them in scalar registers
+    const unsigned long long wo = (unsigned long long)tc * wstep;
+    const unsigned wlo = __builtin_amdgcn_readfirstlane((unsigned)wo), whi = __builtin_amdgcn_readfirstlane((unsigned)(wo >> 32));
+    const char* at = Abase + __builtin_amdgcn_readfirstlane(tc * (int)(BK * sizeof(float)));
+    const char* wt = Wbase + (((unsigned long long)whi << 32) | wlo);
+    Share r;
+#pragma unroll
+    for (int j = 0; j < NA; ++j) r.a[j] = *reinterpret_cast<const float4*>(at + aoff[j]);
+#pragma unroll
+    for (int j = 0; j < NB; ++j) r.b[j] = *reinterpret_cast<const float4*>(wt + boff[j]);
+    return r;
+  };
+  Share set[2];
+  auto fetch = [&](auto P, int tile) { set[decltype(P)::value] = load_share(tile); };
+  // LDS layouts: A tile as [m][BK + 4], W tile as [k][TN] with the two 32-column halves of a 64-column group
+  // swapped in rows with bit 2 set. Matrix instruction i of quarter q takes k = 8q + 4h + i from half-wave h, so a
+  // lane's four A values of a quarter are one 128-bit read of the unpermuted row, and the two half-waves of a W
+  // read (rows 8q + i and 8q + 4 + i) use different banks.
+  float* const adst = As + arow * AST + akq;
+  float* const bdst = Bs + brow * TN + (bnq ^ (((brow >> 2) & 1) << 5));  // rows + 16r have the same bit 2
+  auto stage = [&](auto P, int st) {  // set p -> LDS stage st
+    constexpr int p = decltype(P)::value;
+#pragma unroll
+    for (int j = 0; j < NA; ++j) st4(adst + st * (TM * AST) + 32 * j, set[p].a[j]);
+#pragma unroll
+    for (int j = 0; j < NB; ++j) st4(bdst + st * (BK * TN) + 16 * j * TN, set[p].b[j]);
+  };
+  float av[HK], bv[HK];
+  const float* const asrc = As + (wm + l32) * AST + 4 * h;
+  const float* const bsrc = Bs + 4 * h * TN + ((wn + l32) ^ (h << 5));
+  auto operands = [&](int st) {  // the wave's operands of a whole K step
+#pragma unroll
+    for (int q = 0; q < HK / 4; ++q) {
+      const float4 v = ld4(asrc + st * (TM * AST) + 8 * q);
+      av[4 * q] = v.x; av[4 * q + 1] = v.y; av[4 * q + 2] = v.z; av[4 * q + 3] = v.w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bv[4 * q + i] = bsrc[st * (BK * TN) + (8 * q + i) * TN];
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  auto multiply = [&]() {
+#pragma unroll
+    for (int i = 0; i < HK; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
+  };
+  const int n = n0 + wn + l32;
+  const float bvs = (bias && n < N) ? bias[n] : 0.f;  // requested early: the epilogue does not wait for it
+
+  typedef std::integral_constant<int, 0> P0;
+  typedef std::integral_constant<int, 1> P1;
+  // the matrix instructions touch registers only, so the scheduler would move them across a barrier into the
+  // memory phase and undo the alternation: pin both sides
+  auto phase_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Tile j lives in LDS stage j & 1 and travels through register set j & 1. The two groups run separate
+  // loops with the same number of barriers (1 + 2 * nsteps), so that no value has to be merged between
+  // their code paths.
+  if (g == 0) {
+    // multiplies step k in the first half of iteration k; leads by two tiles: 0 and 1 staged, 2 and 3 in flight
+    fetch(P0(), 0);
+    fetch(P1(), 1);
+    const Share t2 = load_share(2), t3 = load_share(3);  // requested before the first two are waited for
+    stage(P0(), 0);
+    stage(P1(), 1);
+    set[0] = t2;
+    set[1] = t3;
+    phase_barrier();
+    operands(0);
+    auto iteration = [&](auto parity, int k) {
+      typedef decltype(parity) P;
+      multiply();  // step k
+      phase_barrier();
+      operands(1 - P::value);  // step k + 1
+      stage(P(), P::value);    // tile k + 2
+      fetch(P(), k + 4);
+      phase_barrier();
+    };
+    int k = 0;
+    for (; k + 1 < nsteps; k += 2) {
+      iteration(P0(), k);
+      iteration(P1(), k + 1);
+    }
+    if (k < nsteps) iteration(P0(), k);
+  } else {
+    // multiplies step k in the second half of iteration k; leads by one tile: 0 staged, 1 and 2 in flight
+    fetch(P0(), 0);
+    fetch(P1(), 1);
+    const Share t2 = load_share(2);
+    stage(P0(), 0);
+    set[0] = t2;
+    phase_barrier();
+    auto iteration = [&](auto parity, int k) {
+      typedef decltype(parity) P;
+      typedef std::integral_constant<int, 1 - P::value> Q;
+      operands(P::value);      // step k
+      stage(Q(), Q::value);    // tile k + 1
+      fetch(Q(), k + 3);
+      phase_barrier();
+      multiply();  // step k
+      phase_barrier();
+    };
+    int k = 0;
+    for (; k + 1 < nsteps; k += 2) {
+      iteration(P0(), k);
+      iteration(P1(), k + 1);
+    }
+    if (k < nsteps) iteration(P0(), k);
+  }
+
+  if (n < N) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = m0 + wm + (i >> 2) * 8 + h * 4 + (i & 3);
+      if (m < M) {
+        float v = acc[i] + bvs;
+        if (epi == EPI_GELU) v = gelu_ref(v);
+        else if (epi == EPI_RESIDUAL) v += resid[(size_t)m * ldc + n];
+        C[(size_t)m * ldc + n] = v;
+      }
+    }
   }
 }
 
@@ -1157,14 +1361,16 @@ template <int TM, int TN, int BK, bool I8W>
 void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const void* W, int ldw, const float* wscale,
                    const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
   const dim3 grid(cdiv(N, TN), cdiv(M, TM), S);
-  if (S == 1) {
-    gemm_mfma<TM, TN, BK, I8W><<<grid, WG, 0, s>>>(M, N, K, K, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid);
-  } else {
-    // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
-    const int kchunk = (int)cdiv(cdiv(K, S), BK) * BK;
-    gemm_mfma<TM, TN, BK, I8W><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, nullptr, workspace, N, EPI_NONE, nullptr);
-    gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
-  }
+  // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
+  const int kchunk = S == 1 ? K : (int)cdiv(cdiv(K, S), BK) * BK;
+  const bool exact = K % BK == 0;  // then every slice is whole steps (kchunk is a multiple of BK)
+  const float* kb = S == 1 ? bias : nullptr;
+  float* kc = S == 1 ? C : workspace;
+  const int kldc = S == 1 ? ldc : N, kepi = S == 1 ? epi : EPI_NONE;
+  const float* kres = S == 1 ? resid : nullptr;
+  if (exact) gemm_mfma<TM, TN, BK, I8W, true><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
+  else gemm_mfma<TM, TN, BK, I8W, false><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
+  if (S > 1) gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
 }
 
 // 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
@@ -1173,6 +1379,32 @@ void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const vo
 template <bool I8W>
 void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int ldw, const float* wscale, const float* bias,
               float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+  // 64 x 128 tiles of the two-group kernel when, with K split at most 4 ways, they give each of the 256
+  // compute units one workgroup (and at most two)
+  const size_t pp = (size_t)cdiv(M, 64) * cdiv(N, 128);
+  if (!I8W && K % PP_BK == 0 && pp >= 64) {
+    int S = 1;
+    while (workspace && S < 4 && pp * S < 256 && K / (2 * S) >= 128 && (K / (2 * S)) % PP_BK == 0) S *= 2;
+    // whole rounds of 256 workgroups, or nearly: a last round that leaves compute units idle costs as much as a full one
+    const size_t wgs = pp * S, rounds = cdiv(wgs, 256);
+    if (wgs * 100 >= rounds * 256 * 85 && wgs <= 1024) {
+      static const bool raised = [] {
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pingpong<PP_BK>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)PP_LDS) == hipSuccess;
+      }();
+      if (raised) {
+        const dim3 grid(cdiv(N, 128), cdiv(M, 64), S);
+        const float* Wf = static_cast<const float*>(W);
+        if (S == 1) {
+          gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K, A, lda, Wf, ldw, bias, C, ldc, epi, resid);
+        } else {
+          gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K / S, A, lda, Wf, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
+          gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+        }
+        return;
+      }
+    }
+  }
   const bool big = (size_t)cdiv(M, 128) * cdiv(N, 128) >= 512;
   const int t = big ? 128 : 64;
   int S = 1;
