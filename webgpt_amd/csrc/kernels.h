@@ -26,12 +26,22 @@ hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const fl
 // workspace (gemm_workspace_floats(M, N) floats, may be null) enables split-K for
 // shapes with too few output tiles to fill the GPU.
 size_t gemm_workspace_floats(int M, int N);
+// A LayerNormBlock applied to the finished rows of C right after the product (out may not alias C). Where the
+// product ends in a split-K reduction pass, that pass normalises the rows it has just finished.
+struct LnAfter {
+  const float* gamma;
+  const float* beta;
+  float* out;
+  int ldo;
+};
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
-                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
+                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
+                       const LnAfter* ln = nullptr);
 // Same with the packed int8 weights of other/int8-gemm.js (Wq[K, ldwq] words, scale[N]), dequantised inside
 // the kernel; M >= 16.
 hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
-                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s);
+                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
+                          const LnAfter* ln = nullptr);
 
 // int8 weight-only variants: Wq is [K, ldwq] words holding 4 columns each.
 hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,

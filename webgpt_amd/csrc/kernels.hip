@@ -146,6 +146,70 @@ __global__ __launch_bounds__(WG) void gemv_reduce(int M, int N, int S, const flo
   st4(C + (size_t)r * ldc + n0, s);
 }
 
+// gemv_reduce of one row followed by the LayerNorm of that row (layernorm_kernel's arithmetic and order of
+// operations, thread t holding the float4 t, t + WG, ... of the row): C gets the finished row, ln_out its
+// normalisation. One workgroup per row; N a multiple of 4, at most 4 * WG * REDUCE_LN_MAXV.
+constexpr int REDUCE_LN_MAXV = 4;
+__global__ __launch_bounds__(WG) void reduce_ln_kernel(int M, int N, int S, const float* __restrict__ part,
+                                                        const float* __restrict__ bias, float* C, int ldc, int epi,
+                                                        const float* resid, const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta, float* __restrict__ ln_out, int ldo) {
+  __shared__ float sh[NWAVE];
+  const int r = blockIdx.x, n4 = N >> 2;
+  float4 v[REDUCE_LN_MAXV];
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < REDUCE_LN_MAXV; ++j) {
+    const int i = threadIdx.x + j * WG;
+    v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < n4) {
+      const int n0 = 4 * i;
+      float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int sp = 0; sp < S; ++sp) {
+        const float4 p = ld4(part + ((size_t)sp * M + r) * N + n0);
+        a.x += p.x; a.y += p.y; a.z += p.z; a.w += p.w;
+      }
+      if (bias) {
+        const float4 b = ld4(bias + n0);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+      }
+      if (epi == EPI_GELU) {
+        a.x = gelu_ref(a.x); a.y = gelu_ref(a.y); a.z = gelu_ref(a.z); a.w = gelu_ref(a.w);
+      } else if (epi == EPI_RESIDUAL) {
+        const float4 q = ld4(resid + (size_t)r * ldc + n0);
+        a.x += q.x; a.y += q.y; a.z += q.z; a.w += q.w;
+      }
+      st4(C + (size_t)r * ldc + n0, a);
+      v[j] = a;
+      sum += (a.x + a.y) + (a.z + a.w);
+    }
+  }
+  const float mean = block_sum(sum, sh) / (float)N;
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < REDUCE_LN_MAXV; ++j) {
+    if (threadIdx.x + j * WG < n4) {
+      const float a = v[j].x - mean, b = v[j].y - mean, c = v[j].z - mean, d = v[j].w - mean;
+      q += (a * a + b * b) + (c * c + d * d);
+    }
+  }
+  const float var = block_sum(q, sh) / (float)N;
+  const float stdev = sqrtf(var + 1e-5f);
+#pragma unroll
+  for (int j = 0; j < REDUCE_LN_MAXV; ++j) {
+    const int i = threadIdx.x + j * WG;
+    if (i < n4) {
+      const float4 g = ld4(gamma + 4 * i), b = ld4(beta + 4 * i);
+      float4 o;
+      o.x = g.x * ((v[j].x - mean) / stdev) + b.x;
+      o.y = g.y * ((v[j].y - mean) / stdev) + b.y;
+      o.z = g.z * ((v[j].z - mean) / stdev) + b.z;
+      o.w = g.w * ((v[j].w - mean) / stdev) + b.w;
+      st4(ln_out + (size_t)r * ldo + 4 * i, o);
+    }
+  }
+}
+
 // int8 weight-only stage 1 (other/int8-gemm.js:156-210 at M <= 4): a wave reads
 // 64 consecutive words (256 columns) of one row; 4 waves take rows k0+ty, +4, ...
 template <int R>
@@ -1357,9 +1421,22 @@ hipError_t launch_dequant_i8(int K, int N, const int32_t* Wq, int ldwq, const fl
 size_t gemm_workspace_floats(int M, int N) { return (size_t)8 * M * N; }
 
 namespace {
+// Second pass of a split-K product: ordered sum of the S partial matrices, bias, epilogue; with `ln` the
+// LayerNorm of the finished rows in the same kernel.
+void finish_split(int M, int N, int S, const float* workspace, const float* bias, float* C, int ldc, int epi, const float* resid,
+                  const LnAfter* ln, hipStream_t s) {
+  if (ln && (N & 3) == 0 && N <= 4 * WG * REDUCE_LN_MAXV) {
+    reduce_ln_kernel<<<M, WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid, ln->gamma, ln->beta, ln->out, ln->ldo);
+    return;
+  }
+  gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+}
+
 template <int TM, int TN, int BK, bool I8W>
 void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const void* W, int ldw, const float* wscale,
-                   const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+                   const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, const LnAfter* ln,
+                   hipStream_t s) {
   const dim3 grid(cdiv(N, TN), cdiv(M, TM), S);
   // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
   const int kchunk = S == 1 ? K : (int)cdiv(cdiv(K, S), BK) * BK;
@@ -1370,7 +1447,8 @@ void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const vo
   const float* kres = S == 1 ? resid : nullptr;
   if (exact) gemm_mfma<TM, TN, BK, I8W, true><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
   else gemm_mfma<TM, TN, BK, I8W, false><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
-  if (S > 1) gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  if (S > 1) finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, s);
+  else if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
 }
 
 // 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
@@ -1378,7 +1456,7 @@ void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const vo
 // at least 128) until there are two workgroups per compute unit.
 template <bool I8W>
 void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int ldw, const float* wscale, const float* bias,
-              float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+              float* C, int ldc, int epi, const float* resid, float* workspace, const LnAfter* ln, hipStream_t s) {
   // 64 x 128 tiles of the two-group kernel when, with K split at most 4 ways, they give each of the 256
   // compute units one workgroup (and at most two)
   const size_t pp = (size_t)cdiv(M, 64) * cdiv(N, 128);
@@ -1397,9 +1475,10 @@ void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int l
         const float* Wf = static_cast<const float*>(W);
         if (S == 1) {
           gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K, A, lda, Wf, ldw, bias, C, ldc, epi, resid);
+          if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
         } else {
           gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K / S, A, lda, Wf, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
-          gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+          finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, s);
         }
         return;
       }
@@ -1410,26 +1489,28 @@ void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int l
   int S = 1;
   const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
   while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
-  if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, s);
-  else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, s);
+  if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, s);
+  else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, s);
 }
 }  // namespace
 
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
-                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s, const LnAfter* ln) {
   if (M < 16) {
     // too few rows for a matrix-core tile: scalar-FMA tile kernel
     gemm_tile64<<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
+    if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
     return hipGetLastError();
   }
-  run_gemm<false>(M, N, K, A, lda, W, ldw, nullptr, bias, C, ldc, epi, resid, workspace, s);
+  run_gemm<false>(M, N, K, A, lda, W, ldw, nullptr, bias, C, ldc, epi, resid, workspace, ln, s);
   return hipGetLastError();
 }
 
 hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
-                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s) {
+                          const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
+                          const LnAfter* ln) {
   if (M < 16 || (N & 3)) return hipErrorInvalidValue;
-  run_gemm<true>(M, N, K, A, lda, Wq, ldwq, scale, bias, C, ldc, epi, resid, workspace, s);
+  run_gemm<true>(M, N, K, A, lda, Wq, ldwq, scale, bias, C, ldc, epi, resid, workspace, ln, s);
   return hipGetLastError();
 }
 

@@ -88,24 +88,29 @@ static bool parse_name(Model* m, const std::string& name, Slot* slot) {
 }
 
 // C[M,ldc] = epi(A . W + bias) with W fp32 or int8 weight-only.
+// With `ln` the LayerNorm that follows in the forward is applied to the finished rows as part of the product.
 static int linear(Model* m, int M, int N, int K, const float* A, int lda, const LinW& w, const float* bias, float* C,
-                  int ldc, int epi, const float* resid) {
+                  int ldc, int epi, const float* resid, const LnAfter* ln = nullptr) {
   hipStream_t s = rt().stream;
   hipError_t e;
+  bool ln_done = true;
   if (w.q) {
     if (M <= GEMV_MAX_ROWS) {
       e = launch_gemv_kn_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
+      ln_done = false;
     } else if (M >= 16) {
-      e = launch_gemm_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
+      e = launch_gemm_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s, ln);
     } else {
       e = launch_dequant_i8(K, N, w.q, N / 4, w.s, m->dq, N, s);
-      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s);
+      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s, ln);
     }
   } else if (M <= GEMV_MAX_ROWS) {
     e = launch_gemv_kn(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
+    ln_done = false;
   } else {
-    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
+    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s, ln);
   }
+  if (e == hipSuccess && ln && !ln_done) e = launch_layernorm(M, N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo, s);
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "linear layer launch: %s", hipGetErrorString(e));
   return WGPT_OK;
 }
@@ -139,7 +144,8 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
     const LayerW& l = m->layers[li];
     float* Kc = m->kv + ((size_t)li * 2 + 0) * m->ctx * d;
     float* Vc = m->kv + ((size_t)li * 2 + 1) * m->ctx * d;
-    LAUNCH(launch_layernorm(T, d, m->x, d, l.ln1_g, l.ln1_b, m->ln, d, s));
+    // without taps the LayerNorm in front of a product is applied by the product before it (see linear)
+    if (taps || li == 0) LAUNCH(launch_layernorm(T, d, m->x, d, l.ln1_g, l.ln1_b, m->ln, d, s));
     if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
     ++ti;
     if ((rc = linear(m, T, 3 * d, d, m->ln, d, l.attn, l.attn_b, m->qkv, 3 * d, EPI_NONE, nullptr))) return rc;
@@ -150,12 +156,13 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
       if ((rc = tap(m, T, ti, m->tmp))) return rc;
       LAUNCH(launch_residual((size_t)T * d / 4, m->tmp, m->x, m->x, s));
     } else {
-      if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->x, d, EPI_RESIDUAL, m->x))) return rc;
+      const LnAfter ln2 = {l.ln2_g, l.ln2_b, m->ln, d};
+      if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->x, d, EPI_RESIDUAL, m->x, &ln2))) return rc;
     }
     ++ti;
     if (taps && (rc = tap(m, T, ti, m->x))) return rc;
     ++ti;
-    LAUNCH(launch_layernorm(T, d, m->x, d, l.ln2_g, l.ln2_b, m->ln, d, s));
+    if (taps) LAUNCH(launch_layernorm(T, d, m->x, d, l.ln2_g, l.ln2_b, m->ln, d, s));
     if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
     ++ti;
     if ((rc = linear(m, T, hid, d, m->ln, d, l.fc, l.fc_b, m->h, hid, EPI_GELU, nullptr))) return rc;
@@ -164,7 +171,12 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
       if ((rc = tap(m, T, ti, m->tmp))) return rc;
       LAUNCH(launch_residual((size_t)T * d / 4, m->tmp, m->x, m->x, s));
     } else {
-      if ((rc = linear(m, T, d, hid, m->h, hid, l.fc2, l.fc2_b, m->x, d, EPI_RESIDUAL, m->x))) return rc;
+      if (li + 1 < m->L) {
+        const LnAfter ln1 = {m->layers[li + 1].ln1_g, m->layers[li + 1].ln1_b, m->ln, d};
+        if ((rc = linear(m, T, d, hid, m->h, hid, l.fc2, l.fc2_b, m->x, d, EPI_RESIDUAL, m->x, &ln1))) return rc;
+      } else {
+        if ((rc = linear(m, T, d, hid, m->h, hid, l.fc2, l.fc2_b, m->x, d, EPI_RESIDUAL, m->x))) return rc;
+      }
     }
     ++ti;
     if (taps && (rc = tap(m, T, ti, m->x))) return rc;
