@@ -34,14 +34,21 @@ struct LnAfter {
   float* out;
   int ldo;
 };
+// For a product that yields a [M, 3d] q/k/v matrix: the key and value columns of row i also go to row pos0 + i of
+// the head-major cache (launch_kv_append's layout), by the pass that finishes C where there is one.
+struct KvAfter {
+  float* Kc;
+  float* Vc;
+  int d, hs, ctx, pos0;
+};
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
                        float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
-                       const LnAfter* ln = nullptr);
+                       const LnAfter* ln = nullptr, const KvAfter* kv = nullptr);
 // Same with the packed int8 weights of other/int8-gemm.js (Wq[K, ldwq] words, scale[N]), dequantised inside
 // the kernel; M >= 16.
 hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
                           const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
-                          const LnAfter* ln = nullptr);
+                          const LnAfter* ln = nullptr, const KvAfter* kv = nullptr);
 
 // int8 weight-only variants: Wq is [K, ldwq] words holding 4 columns each.
 hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq,

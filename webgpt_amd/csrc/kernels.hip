@@ -121,9 +121,11 @@ __global__ __launch_bounds__(WG) void gemv_kn_partial(int N, int K, const float*
   }
 }
 
+// With kv.Kc set, C is a [M, 3d] q/k/v matrix whose key and value columns also go to the head-major cache
+// (kv_append_kernel's layout).
 __global__ __launch_bounds__(WG) void gemv_reduce(int M, int N, int S, const float* __restrict__ part,
                                                    const float* __restrict__ bias, float* C, int ldc, int epi,
-                                                   const float* resid) {
+                                                   const float* resid, KvAfter kv = KvAfter{nullptr, nullptr, 0, 0, 0, 0}) {
   const int n4 = N >> 2;
   const int idx = blockIdx.x * WG + threadIdx.x;
   if (idx >= M * n4) return;
@@ -144,6 +146,10 @@ __global__ __launch_bounds__(WG) void gemv_reduce(int M, int N, int S, const flo
     s.x += q.x; s.y += q.y; s.z += q.z; s.w += q.w;
   }
   st4(C + (size_t)r * ldc + n0, s);
+  if (kv.Kc && n0 >= kv.d) {
+    const int which = n0 >= 2 * kv.d, c = n0 - (1 + which) * kv.d, h = c / kv.hs, e = c - h * kv.hs;
+    st4((which ? kv.Vc : kv.Kc) + ((size_t)h * kv.ctx + kv.pos0 + r) * kv.hs + e, s);
+  }
 }
 
 // gemv_reduce of one row followed by the LayerNorm of that row (layernorm_kernel's arithmetic and order of
@@ -1424,7 +1430,12 @@ namespace {
 // Second pass of a split-K product: ordered sum of the S partial matrices, bias, epilogue; with `ln` the
 // LayerNorm of the finished rows in the same kernel.
 void finish_split(int M, int N, int S, const float* workspace, const float* bias, float* C, int ldc, int epi, const float* resid,
-                  const LnAfter* ln, hipStream_t s) {
+                  const LnAfter* ln, const KvAfter* kv, hipStream_t s) {
+  if (kv) {
+    gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid, *kv);
+    if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+    return;
+  }
   if (ln && (N & 3) == 0 && N <= 4 * WG * REDUCE_LN_MAXV) {
     reduce_ln_kernel<<<M, WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid, ln->gamma, ln->beta, ln->out, ln->ldo);
     return;
@@ -1433,10 +1444,16 @@ void finish_split(int M, int N, int S, const float* workspace, const float* bias
   if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
 }
 
+// The same two follow-ups after a product that wrote C itself.
+void finish_direct(int M, int N, const float* C, int ldc, const LnAfter* ln, const KvAfter* kv, hipStream_t s) {
+  if (kv) kv_append_kernel<<<M, WG, 0, s>>>(kv->d, kv->hs, kv->ctx, kv->pos0, C, kv->Kc, kv->Vc);
+  if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+}
+
 template <int TM, int TN, int BK, bool I8W>
 void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const void* W, int ldw, const float* wscale,
                    const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, const LnAfter* ln,
-                   hipStream_t s) {
+                   const KvAfter* kv, hipStream_t s) {
   const dim3 grid(cdiv(N, TN), cdiv(M, TM), S);
   // partial sums of the K slices are combined in ascending order by gemv_reduce (deterministic), bias last
   const int kchunk = S == 1 ? K : (int)cdiv(cdiv(K, S), BK) * BK;
@@ -1447,8 +1464,8 @@ void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const vo
   const float* kres = S == 1 ? resid : nullptr;
   if (exact) gemm_mfma<TM, TN, BK, I8W, true><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
   else gemm_mfma<TM, TN, BK, I8W, false><<<grid, WG, 0, s>>>(M, N, K, kchunk, A, lda, W, ldw, wscale, kb, kc, kldc, kepi, kres);
-  if (S > 1) finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, s);
-  else if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+  if (S > 1) finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, kv, s);
+  else finish_direct(M, N, C, ldc, ln, kv, s);
 }
 
 // 128x128 tiles when they alone fill the 256 compute units twice over, else 64x64 (measured
@@ -1456,7 +1473,8 @@ void run_gemm_mfma(int M, int N, int K, int S, const float* A, int lda, const vo
 // at least 128) until there are two workgroups per compute unit.
 template <bool I8W>
 void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int ldw, const float* wscale, const float* bias,
-              float* C, int ldc, int epi, const float* resid, float* workspace, const LnAfter* ln, hipStream_t s) {
+              float* C, int ldc, int epi, const float* resid, float* workspace, const LnAfter* ln, const KvAfter* kv,
+              hipStream_t s) {
   // 64 x 128 tiles of the two-group kernel when, with K split at most 4 ways, they give each of the 256
   // compute units one workgroup (and at most two)
   const size_t pp = (size_t)cdiv(M, 64) * cdiv(N, 128);
@@ -1475,10 +1493,10 @@ void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int l
         const float* Wf = static_cast<const float*>(W);
         if (S == 1) {
           gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K, A, lda, Wf, ldw, bias, C, ldc, epi, resid);
-          if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+          finish_direct(M, N, C, ldc, ln, kv, s);
         } else {
           gemm_pingpong<PP_BK><<<grid, PP_THREADS, PP_LDS, s>>>(M, N, K, K / S, A, lda, Wf, ldw, nullptr, workspace, N, EPI_NONE, nullptr);
-          finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, s);
+          finish_split(M, N, S, workspace, bias, C, ldc, epi, resid, ln, kv, s);
         }
         return;
       }
@@ -1489,28 +1507,29 @@ void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int l
   int S = 1;
   const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
   while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
-  if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, s);
-  else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, s);
+  if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, kv, s);
+  else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, kv, s);
 }
 }  // namespace
 
 hipError_t launch_gemm(int M, int N, int K, const float* A, int lda, const float* W, int ldw, const float* bias,
-                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s, const LnAfter* ln) {
+                       float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s, const LnAfter* ln,
+                       const KvAfter* kv) {
   if (M < 16) {
     // too few rows for a matrix-core tile: scalar-FMA tile kernel
     gemm_tile64<<<dim3(cdiv(N, 64), cdiv(M, 64)), WG, 0, s>>>(M, N, K, A, lda, W, ldw, bias, C, ldc, epi, resid);
-    if (ln) layernorm_kernel<<<M, WG, 0, s>>>(N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo);
+    finish_direct(M, N, C, ldc, ln, kv, s);
     return hipGetLastError();
   }
-  run_gemm<false>(M, N, K, A, lda, W, ldw, nullptr, bias, C, ldc, epi, resid, workspace, ln, s);
+  run_gemm<false>(M, N, K, A, lda, W, ldw, nullptr, bias, C, ldc, epi, resid, workspace, ln, kv, s);
   return hipGetLastError();
 }
 
 hipError_t launch_gemm_i8(int M, int N, int K, const float* A, int lda, const int32_t* Wq, int ldwq, const float* scale,
                           const float* bias, float* C, int ldc, int epi, const float* resid, float* workspace, hipStream_t s,
-                          const LnAfter* ln) {
+                          const LnAfter* ln, const KvAfter* kv) {
   if (M < 16 || (N & 3)) return hipErrorInvalidValue;
-  run_gemm<true>(M, N, K, A, lda, Wq, ldwq, scale, bias, C, ldc, epi, resid, workspace, ln, s);
+  run_gemm<true>(M, N, K, A, lda, Wq, ldwq, scale, bias, C, ldc, epi, resid, workspace, ln, kv, s);
   return hipGetLastError();
 }
 

@@ -90,7 +90,7 @@ static bool parse_name(Model* m, const std::string& name, Slot* slot) {
 // C[M,ldc] = epi(A . W + bias) with W fp32 or int8 weight-only.
 // With `ln` the LayerNorm that follows in the forward is applied to the finished rows as part of the product.
 static int linear(Model* m, int M, int N, int K, const float* A, int lda, const LinW& w, const float* bias, float* C,
-                  int ldc, int epi, const float* resid, const LnAfter* ln = nullptr) {
+                  int ldc, int epi, const float* resid, const LnAfter* ln = nullptr, const KvAfter* kv = nullptr) {
   hipStream_t s = rt().stream;
   hipError_t e;
   bool ln_done = true;
@@ -99,18 +99,21 @@ static int linear(Model* m, int M, int N, int K, const float* A, int lda, const 
       e = launch_gemv_kn_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s);
       ln_done = false;
     } else if (M >= 16) {
-      e = launch_gemm_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s, ln);
+      e = launch_gemm_i8(M, N, K, A, lda, w.q, N / 4, w.s, bias, C, ldc, epi, resid, m->part, s, ln, kv);
     } else {
       e = launch_dequant_i8(K, N, w.q, N / 4, w.s, m->dq, N, s);
-      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s, ln);
+      if (e == hipSuccess) e = launch_gemm(M, N, K, A, lda, m->dq, N, bias, C, ldc, epi, resid, m->part, s, ln, kv);
     }
   } else if (M <= GEMV_MAX_ROWS) {
     e = launch_gemv_kn(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s);
     ln_done = false;
   } else {
-    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s, ln);
+    e = launch_gemm(M, N, K, A, lda, w.w, N, bias, C, ldc, epi, resid, m->part, s, ln, kv);
   }
-  if (e == hipSuccess && ln && !ln_done) e = launch_layernorm(M, N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo, s);
+  if (e == hipSuccess && !ln_done) {  // the matrix-vector kernels take no follow-ups
+    if (kv) e = launch_kv_append(M, kv->d, kv->hs, kv->ctx, kv->pos0, C, kv->Kc, kv->Vc, s);
+    if (e == hipSuccess && ln) e = launch_layernorm(M, N, C, ldc, ln->gamma, ln->beta, ln->out, ln->ldo, s);
+  }
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "linear layer launch: %s", hipGetErrorString(e));
   return WGPT_OK;
 }
@@ -148,8 +151,8 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
     if (taps || li == 0) LAUNCH(launch_layernorm(T, d, m->x, d, l.ln1_g, l.ln1_b, m->ln, d, s));
     if (taps && (rc = tap(m, T, ti, m->ln))) return rc;
     ++ti;
-    if ((rc = linear(m, T, 3 * d, d, m->ln, d, l.attn, l.attn_b, m->qkv, 3 * d, EPI_NONE, nullptr))) return rc;
-    LAUNCH(launch_kv_append(T, d, hs, m->ctx, pos0, m->qkv, Kc, Vc, s));
+    const KvAfter kva = {Kc, Vc, d, hs, m->ctx, pos0};  // the new keys and values join the cache with the product
+    if ((rc = linear(m, T, 3 * d, d, m->ln, d, l.attn, l.attn_b, m->qkv, 3 * d, EPI_NONE, nullptr, nullptr, &kva))) return rc;
     LAUNCH(launch_attention(T, pos0, H, hs, scale, m->qkv, 3 * d, Kc, Vc, (size_t)m->ctx * hs, hs, m->att, d, s));
     if (taps) {
       if ((rc = linear(m, T, d, d, m->att, d, l.proj, l.proj_b, m->tmp, d, EPI_NONE, nullptr))) return rc;
