@@ -47,7 +47,8 @@ def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=253)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed decode steps (default: the configuration's decode length minus the warm-up steps)")
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="gpt2-117m")
     ap.add_argument("--seed", type=int, default=1)
@@ -67,7 +68,9 @@ def main():
     from webgpt_amd._lib import WgptError
 
     cfg = dict(synth.CONFIGS[args.config])
-    if cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
+    if args.steps is None:
+        args.steps = cfg["decode"] - args.warmup
+    if args.steps < 1 or cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
         print(f"bench.py: prompt {cfg['prompt']} + warmup + steps exceeds n_ctx {cfg['n_ctx']}", file=sys.stderr)
         sys.exit(2)
     if args.copy_probe:
