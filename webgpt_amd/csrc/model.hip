@@ -290,7 +290,7 @@ static int setup_persistent(Model* m) {
     static const int tuned[4][7] = {{16, 0, 28, 96, 24, 20, 40},    // d <= 768
                                     {20, 0, 48, 96, 28, 32, 64},    // d = 1024
                                     {20, 0, 48, 96, 4, 20, 40},     // d = 1280
-                                    {40, 0, 48, 96, 32, 40, 40}};   // d = 1600, int8
+                                    {32, 0, 48, 48, 32, 24, 40}};   // d = 1600, int8
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : 3];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
     if (const char* e = getenv("WEBGPT_AMD_POLL_DELAYS")) {
