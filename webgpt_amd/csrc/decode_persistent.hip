@@ -369,14 +369,45 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
   }
 }
 
+// The same row with gamma and beta applied (shapes that cannot fold them into their weights), as a joint
+// effort of the workgroup: every wave derives the statistics itself, wave s % NW finishes segment s
+// and leaves it in xn (an LDS row nobody reads in this phase), and after a barrier every wave takes
+// the finished row from there. Eight waves each applying 2*K parameters from LDS cost two
+// microseconds per LayerNorm at K = 1600.
+template <int K>
+__device__ __forceinline__ void input_row_shared(float4 (&xr)[(K + SEG - 1) / SEG], const float* xs, const float* lnp, float* xn,
+                                                 int wave, int lane) {
+  constexpr int S = (K + SEG - 1) / SEG;
+  const int l4 = opaque(lane) * 4;
+  input_row<K, true, false>(xr, xs, lnp, lane);  // (x - mean) * rstd
+#pragma unroll
+  for (int s2 = 0; s2 < S; ++s2) {
+    if (s2 % NW == wave) {
+      const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
+      float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (in) {
+        const float4 g = *reinterpret_cast<const float4*>(lnp + s2 * SEG + l4);
+        const float4 b = *reinterpret_cast<const float4*>(lnp + K + s2 * SEG + l4);
+        y = make_float4(g.x * xr[s2].x + b.x, g.y * xr[s2].y + b.y, g.z * xr[s2].z + b.z, g.w * xr[s2].w + b.w);
+      }
+      *reinterpret_cast<float4*>(xn + s2 * SEG + l4) = y;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s2 = 0; s2 < S; ++s2) xr[s2] = *reinterpret_cast<const float4*>(xn + s2 * SEG + l4);
+}
+
 // WHOLE phases: the dot products of this wave's columns; lane cc returns the sum of
 // the wave's cc-th column (local column wave + cc * NW), before scale and bias.
 template <class P, bool LNORM, bool AFFINE, class WS>
-__device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const float* lnp, int ncols, int wave, int lane) {
+__device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const float* lnp, int ncols, int wave, int lane,
+                                            float* xn = nullptr) {
   static_assert(P::WHOLE, "phase is not laid out by whole columns");
   // a normalised row is held in registers; a plain one is read from LDS item by item
   float4 xr[LNORM ? P::S : 1];
-  if (LNORM) input_row<P::K, LNORM, AFFINE>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, lane);
+  if constexpr (LNORM && AFFINE) input_row_shared<P::K>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, xn, wave, lane);
+  else if constexpr (LNORM) input_row<P::K, LNORM, AFFINE>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, lane);
   const float* xl = xs + opaque(lane) * 4;
   float val = 0.f;
 #pragma unroll
@@ -636,7 +667,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (DUAL) load_items<PC>(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
         const ColParams cp = col_params<I8>(colp, PH, fc);
-        const float dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane);
+        const float dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1);
         TRACE5(2);
         if (finA) pubA[fc] = finish<I8>(dot, cp);
         __syncthreads();
@@ -831,7 +862,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE(1 + li * 8 + PH);
         if (DUAL) load_items<PE>(wY, slab + a.slab_offE, ncE, wg, wave, lane);
         const ColParams cp = col_params<I8>(colp, PH, fc);
-        const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane);
+        const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1);
         TRACE5(2);
         if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
