@@ -31,7 +31,10 @@ def run(inst, shape):
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 4), (1, 768, 768), (1, 2304, 768), (1, 768, 3072), (1, 72, 100), (2, 64, 64),
                                    (3, 1600, 1600), (4, 384, 1536), (5, 8, 12), (7, 200, 36), (16, 768, 768),
-                                   (128, 2304, 768), (65, 136, 260), (200, 768, 3072), (2048, 4096, 64), (2050, 4104, 40)])
+                                   (128, 2304, 768), (65, 136, 260), (200, 768, 3072), (2048, 4096, 64), (2050, 4104, 40),
+                                   # the two-group kernel: K split four ways, one tile per compute unit, ragged M and N
+                                   # with an odd number of K steps, and the same shape with a ragged K (other kernel)
+                                   (512, 1024, 1024), (512, 4096, 1024), (950, 2056, 96), (950, 2056, 100)])
 def test_fast_matmul(device, M, N, K):
     A, W, b = rnd(M, K), rnd(K, N, scale=0.05), rnd(N)
     inst = FastMatMulBlock.newInstance(M, N, K, init_tensor(A, [M, K]), init_tensor(W, [K, N]), init_tensor(b, [N]))
