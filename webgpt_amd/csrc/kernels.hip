@@ -584,9 +584,7 @@ __global__ __launch_bounds__(WG) void gemm_mfma(int M, int N, int K, int kchunk,
 // unconditional: tiles beyond the K range are fetched from clamped addresses and staged as zeros.
 // ---------------------------------------------------------------------------
 constexpr int PP_THREADS = 512;
-#ifndef PP_BK
-#define PP_BK 32
-#endif
+constexpr int PP_BK = 32;  // K step (64 measured 3-5 % slower)
 constexpr size_t PP_LDS = sizeof(float) * 2 * (64 * (PP_BK + 4) + PP_BK * 128);
 template <int BK>
 __global__ __launch_bounds__(PP_THREADS) void gemm_pingpong(int M, int N, int K, int kchunk, const float* __restrict__ A, int lda,
