@@ -20,6 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+MFMA_FP32_PEAK_FLOPS = 157.3e12  # MI355X dense fp32 matrix
 
 
 def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
@@ -97,6 +98,8 @@ def main():
     prefill_wall_ms = (time.perf_counter() - t0) * 1000.0
     prefill_gpu_ms = gpt.lastGpuMs
     tok = int(np.argmax(logits))
+    T, L, d = len(prompt), cfg["n_layer"], cfg["n_embd"]
+    prefill_flops = 2.0 * T * 12 * L * d * d + 2.0 * L * T * T * d
 
     # warmup steps, then exactly K timed steps, all on the device
     pos = len(prompt)
@@ -156,6 +159,9 @@ def main():
         "prefill_tokens_per_s": round(len(prompt) / (prefill_gpu_ms * 1e-3), 1),
         "prefill_ms": round(prefill_gpu_ms, 3),
         "prefill_wall_ms": round(prefill_wall_ms, 3),
+        # whole prefill (all kernels) against the fp32 MFMA peak: linear-layer flops 2*T*12*L*d^2 + causal attention 2*L*T^2*d
+        "prefill_tflops": round(prefill_flops / (prefill_gpu_ms * 1e-3) / 1e12, 2),
+        "prefill_frac_of_fp32_mfma_peak": round(prefill_flops / (prefill_gpu_ms * 1e-3) / MFMA_FP32_PEAK_FLOPS, 4),
         "host_loop_ms_per_token": {"mean": round(float(np.mean(per_tok)), 4), "p50": round(float(np.median(per_tok)), 4),
                                    "note": "wgpt_decode per token incl. logits read-back over PCIe"} if per_tok else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
