@@ -52,6 +52,9 @@ struct Model {
   bool persist_ok = false;
   PersistentArgs pa{};
   int* perr = nullptr;       // device error word of the persistent kernel
+  // pinned host words (hipHostMalloc): [0] the token of a single-step call on its way to the device,
+  // [1] the error word on its way back, so that a decode call needs one stream synchronisation
+  int32_t* pin = nullptr;
   unsigned epoch = 0;        // last epoch published by earlier launches
 
   hipEvent_t ev0 = nullptr, ev1 = nullptr;

@@ -352,8 +352,8 @@ static int check_persistent(Model* m) {
     }
   }
 #endif
-  int herr = 0;
-  WGPT_HIP(hipMemcpy(&herr, m->perr, sizeof(int), hipMemcpyDeviceToHost));
+  // the error word came back with the call's results (finish_timed)
+  const int herr = m->pin[1];
   if (herr != 0) {
     (void)hipMemset(m->perr, 0, sizeof(int));
     m->persist_ok = false;  // do not trust the exchange buffers again
@@ -366,6 +366,7 @@ static int check_persistent(Model* m) {
 static int finish_timed(Model* m, float* logits) {
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   return WGPT_OK;
@@ -373,6 +374,7 @@ static int finish_timed(Model* m, float* logits) {
 
 static void destroy_model(Model* m) {
   for (void* p : m->allocs) (void)hipFree(p);
+  if (m->pin) (void)hipHostFree(m->pin);
   if (m->ev0) (void)hipEventDestroy(m->ev0);
   if (m->ev1) (void)hipEventDestroy(m->ev1);
   delete m;
@@ -457,6 +459,10 @@ int wgpt_model_finalize(wgpt_model h) {
   if ((rc = dev_alloc(m, T * 4 * d * f, (void**)&m->h))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->V * f, (void**)&m->logits))) return rc;
   if ((rc = dev_alloc(m, T * sizeof(int32_t), (void**)&m->tok_dev))) return rc;
+  if (!m->pin) {
+    WGPT_HIP(hipHostMalloc((void**)&m->pin, 2 * sizeof(int32_t), hipHostMallocDefault));
+    m->pin[0] = m->pin[1] = 0;
+  }
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_samp_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(double), (void**)&m->u_dev))) return rc;
@@ -509,8 +515,8 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode: token id %d outside [0, %d)", token, m->V);
   if (m->pos >= m->ctx) return fail(WGPT_ERR_STATE, "wgpt_decode: context of %d positions is full; prefill a slid window", m->ctx);
-  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
-  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   int rc = m->decode_mode == 1 ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
   if (rc) return rc;
@@ -530,8 +536,8 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   if (steps < 1 || !out_tokens) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: steps >= 1 and out_tokens required");
   if (m->pos + steps > m->ctx)
     return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
-  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
-  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
+  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   const bool persistent = m->decode_mode == 1;
   if (persistent) {
@@ -547,6 +553,7 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_tok_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
   if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   if (persistent) {
@@ -596,6 +603,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   WGPT_HIP(hipMemcpyAsync(out_tokens, in_kernel ? m->out_tok_dev : m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
   if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   if (persistent) {
