@@ -1083,19 +1083,19 @@ __global__ __launch_bounds__(NWV * 64) void attention_mfma_kernel(int Tq, int po
 #pragma unroll
   for (int r = 0; r < 16; ++r) { o0[r] = 0.f; o1[r] = 0.f; }
 
-  // the tile after the current one is already on its way from memory while the current one is multiplied
+  // the tile after the current one is already on its way from memory while the current one is multiplied.
+  // The loads are unconditional (a load under a branch is waited for where the paths join, which would undo the
+  // overlap): rows past the last key repeat it; no query of the block sees them, so their weights are exactly 0
+  // and the repeated values only have to be finite.
   float4 kreg[8], vreg[8];
   auto fetch = [&](int t) {
     const int k0 = t * AMK;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int f = lane + 64 * j, row = f >> 4, c4 = f & 15;
-      kreg[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-      vreg[j] = kreg[j];
-      if (t < te && k0 + row < nkeys) {  // rows past the end are zero
-        kreg[j] = ld4(kbase + (size_t)(k0 + row) * ldkv + 4 * c4);
-        vreg[j] = ld4(vbase + (size_t)(k0 + row) * ldkv + 4 * c4);
-      }
+      const int key = k0 + row < nkeys ? k0 + row : nkeys - 1;
+      kreg[j] = ld4(kbase + (size_t)key * ldkv + 4 * c4);
+      vreg[j] = ld4(vbase + (size_t)key * ldkv + 4 * c4);
     }
   };
   fetch(tb);
