@@ -43,6 +43,30 @@ def test_fast_matmul(device, M, N, K):
     assert close(got, want), worst(got, want)
 
 
+def _dispatch_edge_shapes():
+    """Seeded shapes around the tile counts at which the matmul changes kernel or K split (64x128 tiles in whole
+    rounds of 256 workgroups, 64x64 tiles otherwise), with ragged M, N and K among them."""
+    rng = np.random.default_rng(20240607)
+    shapes = []
+    for tiles in (63, 64, 65, 127, 128, 218, 255, 256, 257, 435, 512, 513, 1023, 1024, 1025):
+        mt = int(rng.integers(2, 17))                      # rows of 64
+        nt = max(1, tiles // mt)                           # columns of 128
+        M = 64 * mt - int(rng.integers(0, 40))
+        N = 128 * nt - 8 * int(rng.integers(0, 8))
+        K = int(rng.choice([32, 96, 100, 128, 256, 260, 512, 1024]))
+        shapes.append((max(M, 5), max(N, 8), K))
+    return shapes
+
+
+@pytest.mark.parametrize("M,N,K", _dispatch_edge_shapes())
+def test_fast_matmul_around_kernel_choices(device, M, N, K):
+    A, W, b = rnd(M, K), rnd(K, N, scale=0.05), rnd(N)
+    inst = FastMatMulBlock.newInstance(M, N, K, init_tensor(A, [M, K]), init_tensor(W, [K, N]), init_tensor(b, [N]))
+    got = run(inst, (M, N))
+    want = ref.matmul_bias(A, W, b)
+    assert close(got, want), worst(got, want)
+
+
 def test_fast_matmul_exact_and_preconditions(device):
     A = RNG.integers(-8, 9, (3, 12)).astype(np.float32)
     W = RNG.integers(-8, 9, (12, 16)).astype(np.float32)
