@@ -200,6 +200,31 @@ def test_larger_shapes_decode_against_oracle(device, name):
     gpt.unloadBuffers()
 
 
+@pytest.mark.parametrize("name,n_layer", [("toy", 3), ("gpt2-117m", 2)])
+def test_persistent_decode_across_the_short_context_limit(device, name, n_layer):
+    # the persistent kernel exists per context range (up to 512 positions, and beyond): steps on both sides of
+    # the limit, and multi-step launches that cross it, against the per-block path
+    cfg = dict(synth.CONFIGS[name])
+    cfg["n_layer"], cfg["n_ctx"] = n_layer, 1024
+    gpt, _ = load(cfg, seed=9, random_ln=True)
+    tokens = synth.tokens(12, "prompt", 540, cfg["vocab_size"])
+    out, ids, sampled = {}, {}, {}
+    u = np.random.default_rng(3).random(16)
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        gpt.prefill(tokens[:505])
+        out[mode] = [gpt.decode(int(tokens[505 + i])) for i in range(14)]       # contexts 506..519
+        lg = gpt.prefill(tokens[:500])
+        ids[mode] = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), 24)]   # one call, contexts 501..524
+        gpt.prefill(tokens[:504])
+        sampled[mode] = [int(t) for t in gpt.decode_sample(int(tokens[504]), len(u), 4, 0.9, u)]
+    for i in range(14):
+        assert close(out[1][i], out[0][i]), (i, worst(out[1][i], out[0][i]))
+    assert ids[0] == ids[1]
+    assert sampled[0] == sampled[1]
+    gpt.unloadBuffers()
+
+
 def test_int8_persistent_decode_against_oracle(device):
     # width of the 1.5B int8 configuration, two layers: persistent int8 decode vs per-block int8 decode vs oracle
     cfg = dict(synth.CONFIGS["gpt2-1.5b-int8"])

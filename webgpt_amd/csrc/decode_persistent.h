@@ -15,6 +15,7 @@ constexpr int PD_SPLIT = 4;      // position slices per head in the attention ph
 constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
 constexpr int PD_COLP = 256;     // floats of one workgroup's column parameters of a layer (4 phases x 32 columns x {bias, scale})
 constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
+constexpr int PD_SHORT_KEYS = 32 * (PD_MAXKV / 2) * PD_SPLIT;  // longest context of the instantiation with half the key batches
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
 // [w*cpw, (w+1)*cpw) of N; a column is S segments ("items") of 256 contraction elements,

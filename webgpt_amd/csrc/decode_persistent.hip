@@ -460,6 +460,60 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
   });
 }
 
+// The long contraction split along K instead (shapes whose whole kernel sits at the register limit, where
+// the compiler fetches a row segment from LDS per item and waits for each): wave w takes segments
+// w, w + NW, ... of every column of the workgroup, so a segment is fetched once for CPW items; the
+// per-wave partial of column c goes to part[c * NW + w] and thread c adds the NW of them in wave order.
+template <class P>
+struct KSplit {
+  static constexpr int SW = (P::S + NW - 1) / NW;  // segments per wave
+  static constexpr int IPW = SW * P::CPW;          // items per wave
+};
+// The loads are unconditional: a wave beyond the last segment re-reads it (and multiplies it with
+// zeros), the slab holds zeros for the columns a workgroup at the ragged end does not have.
+template <class P, class WS, class T>
+__device__ __forceinline__ void load_items_ksplit(WS& ws, const T* __restrict__ slab, int wg, int wave, int lane) {
+  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
+#pragma unroll
+  for (int si = 0; si < KSplit<P>::SW; ++si) {
+    int seg = wave + si * NW;
+    seg = seg < P::S ? seg : P::S - 1;
+#pragma unroll
+    for (int c = 0; c < P::CPW; ++c) ws.w[si * P::CPW + c] = ld_stream(wgbase + (c * P::S + seg) * 64);
+  }
+}
+template <class P, class WS>
+__device__ __forceinline__ void gemv_ksplit(const WS& ws, const float* xs, float* part, int wave, int lane) {
+  const float* xl = xs + opaque(lane) * 4;
+  float acc[P::CPW];
+#pragma unroll
+  for (int c = 0; c < P::CPW; ++c) acc[c] = 0.f;
+#pragma unroll
+  for (int si = 0; si < KSplit<P>::SW; ++si) {
+    const int seg = wave + si * NW;
+    const int segc = seg < P::S ? seg : P::S - 1;
+    float4 x = *reinterpret_cast<const float4*>(xl + segc * SEG);
+    if (seg >= P::S) x = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int c = 0; c < P::CPW; ++c) {
+      const float4 w = to_float4(ws.w[si * P::CPW + c]);
+      acc[c] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < P::CPW; ++c) {
+    const float r = wave_sum(acc[c]);
+    if (lane == 0) part[c * NW + wave] = r;
+  }
+}
+template <class P>
+__device__ __forceinline__ float column_sum_ksplit(const float* part, int c) {
+  float s = 0.f;
+#pragma unroll
+  for (int v = 0; v < NW; ++v) s += part[c * NW + v];
+  return s;
+}
+
 // Second MLP matrix: either layout. Whole columns leave residual + column in pubE;
 // split columns leave per-wave partials in part (finished after the barrier).
 template <class P, bool I8, class WS>
@@ -527,8 +581,9 @@ struct Phases {
   typedef Phase<3 * C::D, C::D, true> A;    // c_attn
   typedef Phase<C::D, C::D, true> Cc;       // attention c_proj
   typedef Phase<C::HID, C::D, true> Dd;     // c_fc
-  typedef Phase<C::D, C::HID, C::I8> E;      // mlp c_proj: whole columns only where an item is one register (int8)
-  static constexpr int MAXI = cmax(cmax(A::IPW, Dd::IPW), cmax(Cc::IPW, E::IPW));
+  typedef Phase<C::D, C::HID, false> E;     // mlp c_proj
+  static constexpr bool EKS = C::I8;        // ... split along the contraction (see KSplit)
+  static constexpr int MAXI = cmax(cmax(A::IPW, Dd::IPW), cmax(Cc::IPW, EKS ? KSplit<E>::IPW : E::IPW));
   // Two register sets (c_attn and c_fc in one, the two projections in the other) let a
   // phase's weights be requested a whole phase ahead, right after the poll of the
   // phase before it; affordable while a set is at most 32 registers.
@@ -545,7 +600,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   typedef typename PS::Dd PD;
   typedef typename PS::E PE;
   constexpr int D = C::D, HS = C::HS, H = C::H, HID = C::HID, SPLIT = C::SPLIT, MAXI = PS::MAXI;
-  constexpr bool DUAL = PS::DUAL, I8 = C::I8;
+  constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS;
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
@@ -586,6 +641,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   const int fc = wave + lane * NW;
   const bool finA = lane < PA::CW && fc < ncA, finC = lane < PC::CW && fc < ncC, finD = lane < PD::CW && fc < ncD;
   const bool finE = lane < PE::CW && fc < ncE;
+  // request of the second MLP matrix's share
+  auto load_e = [&](auto& ws, const auto* slabE) {
+    if constexpr (EKS) load_items_ksplit<PE>(ws, slabE, wg, wave, lane);
+    else load_items<PE>(ws, slabE, ncE, wg, wave, lane);
+  };
 
   // attention role: head and slice of the positions; threads form 32 key groups
   // (tid >> 4) of 16 lanes (tid & 15)
@@ -860,7 +920,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) load_items<PE>(wY, slab + a.slab_offE, ncE, wg, wave, lane);
+        if (DUAL) load_e(wY, slab + a.slab_offE);
         const ColParams cp = col_params<I8>(colp, PH, fc);
         const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1);
         TRACE5(2);
@@ -869,7 +929,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         ++ep;
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
         TRACE5(4);
-        if (!DUAL) load_items<PE>(wY, slab + a.slab_offE, ncE, wg, wave, lane);
+        if (!DUAL) load_e(wY, slab + a.slab_offE);
         TRACE5(5);
       }
 
@@ -896,12 +956,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE(1 + li * 8 + PH);
         if (DUAL) request_next();
         const ColParams cpe = col_params<I8>(colp, PH, tid);  // split columns: thread c finishes local column c
-        phase_e<PE, I8>(wY, xs1, part, pubC, pubE, colp, ncE, finE, fc, wave, lane);
+        if constexpr (EKS) gemv_ksplit<PE>(wY, xs1, part, wave, lane);
+        else phase_e<PE, I8>(wY, xs1, part, pubC, pubE, colp, ncE, finE, fc, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
         if (tid < ncE) {  // model.js:205
-          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(column_sum<PE>(part, tid), cpe);
+          const float dot = EKS ? column_sum_ksplit<PE>(part, tid) : column_sum<PE>(part, tid);
+          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(dot, cpe);
           publish(a.bufR2 + wg * PE::CPW + tid, r2, ep);
         }
         TRACE5(4);
@@ -1233,22 +1295,33 @@ size_t lds_bytes_of() {
   return need > one_per_cu ? need : one_per_cu;
 }
 
-template <class C>
-hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
+template <class C, int MAXKV>
+hipError_t launch_kv(const PersistentArgs& a, hipStream_t s) {
   const size_t lds_bytes = lds_bytes_of<C>();
   static bool enabled = false;  // dynamic LDS size already raised for the two instantiations
   if (!enabled) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, PD_MAXKV, false>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, MAXKV, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, PD_MAXKV, true>),
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_persistent_kernel<C, MAXKV, true>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
     enabled = true;
   }
-  if (a.top_k > 1) decode_persistent_kernel<C, PD_MAXKV, true><<<PD_GRID, NT, lds_bytes, s>>>(a);
-  else decode_persistent_kernel<C, PD_MAXKV, false><<<PD_GRID, NT, lds_bytes, s>>>(a);
+  if (a.top_k > 1) decode_persistent_kernel<C, MAXKV, true><<<PD_GRID, NT, lds_bytes, s>>>(a);
+  else decode_persistent_kernel<C, MAXKV, false><<<PD_GRID, NT, lds_bytes, s>>>(a);
   return hipGetLastError();
+}
+
+// A launch whose last step sees at most half of the longest context runs the instantiation with half
+// the key/value registers (32 fewer float4 per lane: the shapes at the register limit spill less, the
+// others schedule more freely).
+template <class C>
+hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
+  const int keys = a.pos0 + a.nsteps;  // positions the last step attends to
+  if (keys > 32 * PD_MAXKV * PD_SPLIT) return hipErrorInvalidValue;
+  if (keys <= PD_SHORT_KEYS) return launch_kv<C, PD_MAXKV / 2>(a, s);
+  return launch_kv<C, PD_MAXKV>(a, s);
 }
 
 }  // namespace

@@ -335,6 +335,20 @@ static int decode_persistent(Model* m, int steps, int top_k = 1, double temperat
   a.ebase = m->epoch;
   a.pos0 = m->pos;
   a.nsteps = steps;
+  // steps that attend to at most PD_SHORT_KEYS positions run the instantiation with half the key/value
+  // registers; a run that crosses that context length is two launches, the second taking its first
+  // token from the ids the first one wrote
+  const int short_steps = PD_SHORT_KEYS - m->pos;
+  if (short_steps > 0 && short_steps < steps) {
+    a.nsteps = short_steps;
+    LAUNCH(launch_decode_persistent(a, rt().stream));
+    a.ebase += per_step * (unsigned)short_steps;
+    a.pos0 += short_steps;
+    a.tok = a.out_tok + short_steps - 1;
+    a.out_tok += short_steps;
+    if (a.u) a.u += short_steps;
+    a.nsteps = steps - short_steps;
+  }
   LAUNCH(launch_decode_persistent(a, rt().stream));
   m->epoch += per_step * (unsigned)steps;
   return WGPT_OK;
