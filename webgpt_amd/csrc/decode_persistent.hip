@@ -267,37 +267,111 @@ __device__ __forceinline__ void zero_item(int& v) { v = 0; }
 __device__ __forceinline__ float4 to_float4(const float4& v) { return v; }
 __device__ __forceinline__ float4 to_float4(int v) { return bytes_to_float4(v); }
 
-// Requests this wave's items of the workgroup's slab share into registers; item
-// j = c * S + seg of the workgroup is 64 consecutive lanes' worth (a float4, or one
-// word of four int8, per lane) of segment seg of local column c. `ncols` is the
-// number of columns this workgroup finishes (CPW except at the ragged end).
-template <class P, class WS, class T>
-__device__ __forceinline__ void load_items(WS& ws, const T* __restrict__ slab, int ncols, int wg, int wave, int lane) {
-  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
-  if (P::WHOLE) {
-#pragma unroll
-    for (int cc = 0; cc < P::CW; ++cc) {
+// f(std::integral_constant<int, i>) for i = 0 .. N-1.
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>()), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>());
+}
+
+template <class P>
+struct KSplit {
+  static constexpr int SW = (P::S + NW - 1) / NW;  // segments per wave
+  static constexpr int IPW = SW * P::CPW;          // items per wave
+};
+
+// Layouts of a wave's share of a phase: whole columns, runs of consecutive items, segments of every column.
+enum { LAY_WHOLE = 0, LAY_RUNS = 1, LAY_KSPLIT = 2 };
+
+// Requests this wave's items of the workgroup's slab share into registers, one item per call; item
+// j = c * S + seg of the workgroup is 64 consecutive lanes' worth (a float4, or one word of four int8,
+// per lane) of segment seg of local column c. `ncols` is the number of columns this workgroup
+// finishes (CPW except at the ragged end). A call costs the wave the time the memory pipeline takes
+// to accept the request (several clocks per request and wave, the eight waves queueing for one
+// pipeline), so the requests of the next phase are dealt out between the dot products of the current
+// one instead of standing in front of them.
+template <class P, int LAYOUT, class WS, class T>
+struct ItemLoader {
+  static constexpr int N = LAYOUT == LAY_KSPLIT ? KSplit<P>::IPW : P::IPW;
+  WS& ws;
+  const T* wgbase;  // this lane's word of the workgroup's first item
+  int ncols, wave;
+  __device__ __forceinline__ ItemLoader(WS& ws_, const T* slab, int ncols_, int wg, int wave_, int lane)
+      : ws(ws_), wgbase(slab + (size_t)wg * P::ITEMS * 64 + opaque(lane)), ncols(ncols_), wave(wave_) {}
+  template <int I>
+  __device__ __forceinline__ void item() const {
+    if constexpr (LAYOUT == LAY_WHOLE) {
+      constexpr int cc = I / P::S, seg = I % P::S;
       const int c = wave + cc * NW;
-#pragma unroll
-      for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
-      if (c < (P::RAGGED ? ncols : P::CPW)) {
-#pragma unroll
-        for (int seg = 0; seg < P::S; ++seg) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);
+      if constexpr (!P::RAGGED && P::CPW % NW == 0) {
+        ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
+      } else {
+        zero_item(ws.w[I]);
+        if (c < (P::RAGGED ? ncols : P::CPW)) ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
       }
+    } else if constexpr (LAYOUT == LAY_RUNS) {
+      // unconditional: what lies beyond the share re-reads its last item and is never used
+      int j = wave * P::IPW + I;
+      j = j < P::ITEMS ? j : P::ITEMS - 1;
+      ws.w[I] = ld_stream(wgbase + j * 64);
+    } else {
+      // unconditional: a wave beyond the last segment re-reads it (and multiplies it with zeros), the
+      // slab holds zeros for the columns a workgroup at the ragged end does not have
+      constexpr int si = I / P::CPW, c = I % P::CPW;
+      int seg = wave + si * NW;
+      seg = seg < P::S ? seg : P::S - 1;
+      ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
     }
-  } else {
-    const int nitems = ncols * P::S;
-    for_wave(wave, [&](auto W) {
-      constexpr int J0 = decltype(W)::value * P::IPW;
+  }
+  // the items of slot J when the N requests are dealt out over NS slots
+  template <int J, int NS>
+  __device__ __forceinline__ void slot() const {
+    constexpr int B = J * N / NS, E = (J + 1) * N / NS;
+    static_for<E - B>([&](auto k) { this->template item<B + decltype(k)::value>(); });
+  }
+  // All of them at once (the code of a run of requests is shorter than that of the same requests one by one).
+  __device__ __forceinline__ void all() const {
+    if constexpr (LAYOUT == LAY_WHOLE) {
 #pragma unroll
-      for (int i = 0; i < P::IPW; ++i) {
-        zero_item(ws.w[i]);
-        if (J0 + i < P::ITEMS) {
-          if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
+      for (int cc = 0; cc < P::CW; ++cc) {
+        const int c = wave + cc * NW;
+#pragma unroll
+        for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
+        if (c < (P::RAGGED ? ncols : P::CPW)) {
+#pragma unroll
+          for (int seg = 0; seg < P::S; ++seg) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);
         }
       }
-    });
+    } else if constexpr (LAYOUT == LAY_RUNS) {
+      const int nitems = ncols * P::S;
+      for_wave(wave, [&](auto W) {
+        constexpr int J0 = decltype(W)::value * P::IPW;
+#pragma unroll
+        for (int i = 0; i < P::IPW; ++i) {
+          zero_item(ws.w[i]);
+          if (J0 + i < P::ITEMS) {
+            if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
+          }
+        }
+      });
+    } else {
+      static_for<N>([&](auto k) { this->template item<decltype(k)::value>(); });
+    }
   }
+};
+
+// What a dot-product loop calls after item J of its NS when nothing is to be requested.
+struct NoRequests {
+  template <int J, int NS>
+  __device__ __forceinline__ void slot() const {}
+};
+// Keeps the requests where they were written: the scheduler would otherwise move them all to the front.
+template <class R>
+__device__ __forceinline__ void pin_requests() {
+  if constexpr (!std::is_same<R, NoRequests>::value) __builtin_amdgcn_sched_barrier(0);
 }
 
 // LayerNorm parameters travel global memory -> registers (requested with the weights
@@ -370,60 +444,106 @@ __device__ __forceinline__ void input_row(float4 (&xr)[(K + SEG - 1) / SEG], con
 }
 
 // The same row with gamma and beta applied (shapes that cannot fold them into their weights), as a joint
-// effort of the workgroup: every wave derives the statistics itself, wave s % NW finishes segment s
-// and leaves it in xn (an LDS row nobody reads in this phase), and after a barrier every wave takes
-// the finished row from there. Eight waves each applying 2*K parameters from LDS cost two
-// microseconds per LayerNorm at K = 1600.
+// effort of the workgroup: thread t owns float4 t of the row. Each wave sums its 256 elements and their
+// squared distances from the wave's own mean; after a barrier every thread merges the NW pairs the same
+// way (mean = sum of sums / K; sum of squares about it = sum_w q_w + n_w (m_w - mean)^2, the two-pass
+// result without a second exchange), finishes its float4 and leaves it in xn (an LDS row nobody reads in
+// this phase); after a second barrier every wave takes the finished row from there. `red` is 2 * NW
+// floats of LDS scratch. (Every wave deriving the statistics of the whole row and re-reading 2*K
+// parameters cost three microseconds per LayerNorm at K = 1600.)
 template <int K>
 __device__ __forceinline__ void input_row_shared(float4 (&xr)[(K + SEG - 1) / SEG], const float* xs, const float* lnp, float* xn,
-                                                 int wave, int lane) {
+                                                 float* red, int wave, int lane) {
   constexpr int S = (K + SEG - 1) / SEG;
-  const int l4 = opaque(lane) * 4;
-  input_row<K, true, false>(xr, xs, lnp, lane);  // (x - mean) * rstd
-#pragma unroll
-  for (int s2 = 0; s2 < S; ++s2) {
-    if (s2 % NW == wave) {
-      const bool in = s2 * SEG + SEG <= K || s2 * SEG + lane * 4 < K;
-      float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (in) {
-        const float4 g = *reinterpret_cast<const float4*>(lnp + s2 * SEG + l4);
-        const float4 b = *reinterpret_cast<const float4*>(lnp + K + s2 * SEG + l4);
-        y = make_float4(g.x * xr[s2].x + b.x, g.y * xr[s2].y + b.y, g.z * xr[s2].z + b.z, g.w * xr[s2].w + b.w);
-      }
-      *reinterpret_cast<float4*>(xn + s2 * SEG + l4) = y;
-    }
+  static_assert(K % 4 == 0 && S * 64 <= NT, "a thread owns one float4 of the row");
+  const int t = opaque(threadIdx.x);
+  const bool own = t < K / 4;
+  const int tc = t < S * 64 ? t : S * 64 - 1;  // threads beyond the row read its zero padding
+  const float4 x = reinterpret_cast<const float4*>(xs)[tc];
+  int nw = K - wave * SEG;  // elements of the row in this wave
+  nw = nw < 0 ? 0 : (nw > SEG ? SEG : nw);
+  const float sw = wave_sum((x.x + x.y) + (x.z + x.w));
+  const float mw = nw > 0 ? sw * (1.0f / (float)nw) : 0.f;
+  const float dx = x.x - mw, dy = x.y - mw, dz = x.z - mw, dw = x.w - mw;
+  const float qw = wave_sum(own ? (dx * dx + dy * dy) + (dz * dz + dw * dw) : 0.f);
+  if (lane == 0) {
+    red[wave] = sw;
+    red[NW + wave] = qw;
   }
   __syncthreads();
+  float sums[NW], qs[NW];
+#pragma unroll
+  for (int v = 0; v < NW; v += 4) {
+    *reinterpret_cast<float4*>(sums + v) = *reinterpret_cast<const float4*>(red + v);
+    *reinterpret_cast<float4*>(qs + v) = *reinterpret_cast<const float4*>(red + NW + v);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int v = 0; v < NW; ++v) total += sums[v];
+  const float mean = total * (1.0f / (float)K);
+  float m2 = 0.f;
+#pragma unroll
+  for (int v = 0; v < NW; ++v) {
+    const int nv = K - v * SEG < 0 ? 0 : (K - v * SEG > SEG ? SEG : K - v * SEG);
+    if (nv > 0) {
+      const float d = sums[v] * (1.0f / (float)nv) - mean;
+      m2 += qs[v] + (float)nv * (d * d);
+    }
+  }
+  const float rstd = fast_rsqrt(m2 * (1.0f / (float)K) + 1e-5f);
+  if (t < S * 64) {
+    float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (own) {
+      const float4 g = reinterpret_cast<const float4*>(lnp)[t];
+      const float4 b = reinterpret_cast<const float4*>(lnp + K)[t];
+      y = make_float4(g.x * ((x.x - mean) * rstd) + b.x, g.y * ((x.y - mean) * rstd) + b.y,
+                      g.z * ((x.z - mean) * rstd) + b.z, g.w * ((x.w - mean) * rstd) + b.w);
+    }
+    reinterpret_cast<float4*>(xn)[t] = y;
+  }
+  __syncthreads();
+  const int l4 = opaque(lane) * 4;
 #pragma unroll
   for (int s2 = 0; s2 < S; ++s2) xr[s2] = *reinterpret_cast<const float4*>(xn + s2 * SEG + l4);
 }
 
 // WHOLE phases: the dot products of this wave's columns; lane cc returns the sum of
-// the wave's cc-th column (local column wave + cc * NW), before scale and bias.
-template <class P, bool LNORM, bool AFFINE, class WS>
+// the wave's cc-th column (local column wave + cc * NW), before scale and bias. `next` requests
+// its items between the items of this phase.
+template <class P, bool LNORM, bool AFFINE, class WS, class R = NoRequests>
 __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const float* lnp, int ncols, int wave, int lane,
-                                            float* xn = nullptr) {
+                                            float* xn = nullptr, float* red = nullptr, const R& next = R()) {
   static_assert(P::WHOLE, "phase is not laid out by whole columns");
   // a normalised row is held in registers; a plain one is read from LDS item by item
   float4 xr[LNORM ? P::S : 1];
-  if constexpr (LNORM && AFFINE) input_row_shared<P::K>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, xn, wave, lane);
+  if constexpr (LNORM && AFFINE) input_row_shared<P::K>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, xn, red, wave, lane);
   else if constexpr (LNORM) input_row<P::K, LNORM, AFFINE>(reinterpret_cast<float4(&)[(P::K + SEG - 1) / SEG]>(xr), xs, lnp, lane);
   const float* xl = xs + opaque(lane) * 4;
   float val = 0.f;
-#pragma unroll
-  for (int cc = 0; cc < P::CW; ++cc) {
-    if (wave + cc * NW < (P::RAGGED ? ncols : P::CPW)) {
-      float acc = 0.f;
-#pragma unroll
-      for (int seg = 0; seg < P::S; ++seg) {
-        const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
-        const float4 w = to_float4(ws.w[cc * P::S + seg]);
-        acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
-      }
+  static_for<P::CW>([&](auto CC) {
+    constexpr int cc = decltype(CC)::value;
+    const bool valid = wave + cc * NW < (P::RAGGED ? ncols : P::CPW);
+    float acc = 0.f;
+    auto item = [&](auto SG) {
+      constexpr int seg = decltype(SG)::value;
+      const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
+      const float4 w = to_float4(ws.w[cc * P::S + seg]);
+      acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+    };
+    if constexpr (std::is_same<R, NoRequests>::value) {
+      if (valid) static_for<P::S>(item);
+    } else {
+      static_for<P::S>([&](auto SG) {
+        if (valid) item(SG);
+        next.template slot<cc * P::S + decltype(SG)::value, P::CW * P::S>();
+        pin_requests<R>();
+      });
+    }
+    if (valid) {
       const float r = wave_sum(acc);
       val = lane == cc ? r : val;
     }
-  }
+  });
   return val;
 }
 
@@ -431,8 +551,9 @@ __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const
 // code exists once per wave with every index a constant: a phase is short, and what
 // it costs is instruction count (a runtime-indexed single copy measured 5-15 %
 // slower at d = 1280 and 1600).
-template <class P, class WS>
-__device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float* part, int ncols, int wave, int lane) {
+template <class P, class WS, class R = NoRequests>
+__device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float* part, int ncols, int wave, int lane,
+                                           const R& next = R()) {
   static_assert(!P::WHOLE, "phase is laid out by whole columns");
   constexpr int S = P::S;
   const float* xl = xs + opaque(lane) * 4;
@@ -441,11 +562,11 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
     constexpr int WV = decltype(W)::value;
     constexpr int J0 = WV * P::IPW;
     float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < P::IPW; ++i) {
-      if (J0 + i < P::ITEMS) {
+    static_for<P::IPW>([&](auto II) {
+      constexpr int i = decltype(II)::value;
+      if constexpr (J0 + i < P::ITEMS) {
         if (!P::RAGGED || J0 + i < nitems) {
-          const int seg = (J0 + i) % S, col = (J0 + i) / S;
+          constexpr int seg = (J0 + i) % S, col = (J0 + i) / S;
           const float4 x = *reinterpret_cast<const float4*>(xl + seg * SEG);
           const float4 w = to_float4(ws.w[i]);
           acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
@@ -456,7 +577,9 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
           }
         }
       }
-    }
+      next.template slot<i, P::IPW>();
+      pin_requests<R>();
+    });
   });
 }
 
@@ -464,42 +587,26 @@ __device__ __forceinline__ void gemv_split(const WS& ws, const float* xs, float*
 // the compiler fetches a row segment from LDS per item and waits for each): wave w takes segments
 // w, w + NW, ... of every column of the workgroup, so a segment is fetched once for CPW items; the
 // per-wave partial of column c goes to part[c * NW + w] and thread c adds the NW of them in wave order.
-template <class P>
-struct KSplit {
-  static constexpr int SW = (P::S + NW - 1) / NW;  // segments per wave
-  static constexpr int IPW = SW * P::CPW;          // items per wave
-};
-// The loads are unconditional: a wave beyond the last segment re-reads it (and multiplies it with
-// zeros), the slab holds zeros for the columns a workgroup at the ragged end does not have.
-template <class P, class WS, class T>
-__device__ __forceinline__ void load_items_ksplit(WS& ws, const T* __restrict__ slab, int wg, int wave, int lane) {
-  const T* wgbase = slab + (size_t)wg * P::ITEMS * 64 + opaque(lane);
-#pragma unroll
-  for (int si = 0; si < KSplit<P>::SW; ++si) {
-    int seg = wave + si * NW;
-    seg = seg < P::S ? seg : P::S - 1;
-#pragma unroll
-    for (int c = 0; c < P::CPW; ++c) ws.w[si * P::CPW + c] = ld_stream(wgbase + (c * P::S + seg) * 64);
-  }
-}
-template <class P, class WS>
-__device__ __forceinline__ void gemv_ksplit(const WS& ws, const float* xs, float* part, int wave, int lane) {
+template <class P, class WS, class R = NoRequests>
+__device__ __forceinline__ void gemv_ksplit(const WS& ws, const float* xs, float* part, int wave, int lane, const R& next = R()) {
   const float* xl = xs + opaque(lane) * 4;
   float acc[P::CPW];
 #pragma unroll
   for (int c = 0; c < P::CPW; ++c) acc[c] = 0.f;
-#pragma unroll
-  for (int si = 0; si < KSplit<P>::SW; ++si) {
+  static_for<KSplit<P>::SW>([&](auto SI) {
+    constexpr int si = decltype(SI)::value;
     const int seg = wave + si * NW;
     const int segc = seg < P::S ? seg : P::S - 1;
     float4 x = *reinterpret_cast<const float4*>(xl + segc * SEG);
     if (seg >= P::S) x = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int c = 0; c < P::CPW; ++c) {
+    static_for<P::CPW>([&](auto CI) {
+      constexpr int c = decltype(CI)::value;
       const float4 w = to_float4(ws.w[si * P::CPW + c]);
       acc[c] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
-    }
-  }
+      next.template slot<si * P::CPW + c, KSplit<P>::IPW>();
+      pin_requests<R>();
+    });
+  });
 #pragma unroll
   for (int c = 0; c < P::CPW; ++c) {
     const float r = wave_sum(acc[c]);
@@ -512,20 +619,6 @@ __device__ __forceinline__ float column_sum_ksplit(const float* part, int c) {
 #pragma unroll
   for (int v = 0; v < NW; ++v) s += part[c * NW + v];
   return s;
-}
-
-// Second MLP matrix: either layout. Whole columns leave residual + column in pubE;
-// split columns leave per-wave partials in part (finished after the barrier).
-template <class P, bool I8, class WS>
-__device__ __forceinline__ void phase_e(const WS& ws, const float* xs, float* part, const float* pubC, float* pubE,
-                                        const float* colp, int ncols, bool fin, int fc, int wave, int lane) {
-  if constexpr (P::WHOLE) {
-    const ColParams cp = col_params<I8>(colp, PH_FC2, fc);
-    const float dot = gemv_whole<P, false, false>(ws, xs, nullptr, ncols, wave, lane);
-    if (fin) pubE[fc] = pubC[fc] + finish<I8>(dot, cp);
-  } else {
-    gemv_split<P>(ws, xs, part, ncols, wave, lane);
-  }
 }
 
 // Sum of the per-wave partials of local column c, in ascending wave order.
@@ -588,6 +681,11 @@ struct Phases {
   // phase's weights be requested a whole phase ahead, right after the poll of the
   // phase before it; affordable while a set is at most 32 registers.
   static constexpr bool DUAL = MAXI * (C::I8 ? 1 : 4) <= 32;
+  // With two sets the next phase's requests stand either in front of the current phase's work (its
+  // LayerNorm and dot products then wait until the memory pipeline has accepted them) or between
+  // its dot products (they then reach memory later, and the next poll, whose answer returns in
+  // order behind them, may see its words late). Short phases want the first, long ones the second.
+  static constexpr bool SPREAD = DUAL && C::I8;
 };
 
 // SAMPLE: top-k selection and sampling in the kernel (top_k in 2..PD_TOPK); the arg-max kernel
@@ -600,7 +698,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   typedef typename PS::Dd PD;
   typedef typename PS::E PE;
   constexpr int D = C::D, HS = C::HS, H = C::H, HID = C::HID, SPLIT = C::SPLIT, MAXI = PS::MAXI;
-  constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS;
+  constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS, SPREAD = PS::SPREAD;
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
@@ -618,11 +716,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float* attp = lnp + 2 * D;   // [ATTP]
   float* part = attp + ATTP;   // [PART]
   float* qkv_s = part + PART;  // [3*HS]
+  static_assert(FOLD || (XS0 + XS1 + 2 * D + ATTP) % 4 == 0, "part is read as float4 by the cooperative LayerNorm");
   float* pubA = qkv_s + 3 * HS;   // [PA::CPW] finished c_attn columns
   float* pubC = pubA + PA::CPW;   // [PC::CPW] residual stream after the attention projection
   float* pubD = pubC + PC::CPW;   // [PD::CPW] finished c_fc columns
-  float* pubE = pubD + PD::CPW;   // [PE::CPW] residual stream after the MLP (whole-column layout only)
-  float* colp = pubE + PE::CPW;   // [8 * LPW] biases and int8 column scales of this workgroup's columns of the layer
+  float* colp = pubD + PD::CPW + PE::CPW;   // [8 * LPW] biases and int8 column scales of this workgroup's columns of the layer
   static_assert(PA::CPW <= LPW && PC::CPW <= LPW && PD::CPW <= LPW && PE::CPW <= LPW, "a phase has more columns per workgroup than colp holds");
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
@@ -640,12 +738,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // local column this lane finishes (lane cc of wave v: column v + cc * NW)
   const int fc = wave + lane * NW;
   const bool finA = lane < PA::CW && fc < ncA, finC = lane < PC::CW && fc < ncC, finD = lane < PD::CW && fc < ncD;
-  const bool finE = lane < PE::CW && fc < ncE;
-  // request of the second MLP matrix's share
-  auto load_e = [&](auto& ws, const auto* slabE) {
-    if constexpr (EKS) load_items_ksplit<PE>(ws, slabE, wg, wave, lane);
-    else load_items<PE>(ws, slabE, ncE, wg, wave, lane);
-  };
 
   // attention role: head and slice of the positions; threads form 32 key groups
   // (tid >> 4) of 16 lanes (tid & 15)
@@ -660,6 +752,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float4 lnreg[NLN];
   typedef typename std::conditional<I8, int, float4>::type Item;
   const Item* slabs = reinterpret_cast<const Item*>(a.slabs);
+  typedef ItemLoader<PA, LAY_WHOLE, WS, Item> LoadA;
+  typedef ItemLoader<PC, LAY_WHOLE, WS, Item> LoadC;
+  typedef ItemLoader<PD, LAY_WHOLE, WS, Item> LoadD;
+  typedef ItemLoader<PE, EKS ? LAY_KSPLIT : LAY_RUNS, WS, Item> LoadE;
   float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
   int tok = a.tok[0];
@@ -676,7 +772,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     if (t < PD_COLP) colp[t] = preg;
   };
   request_params(0);
-  load_items<PA>(wX, slabs, ncA, wg, wave, lane);
+  LoadA(wX, slabs, ncA, wg, wave, lane).all();
   deposit_params();
   // FOLD: only the final LayerNorm has parameters, and they stay in lnp for good
   if (FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
@@ -724,17 +820,20 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) load_items<PC>(wY, slab + a.slab_offC, ncC, wg, wave, lane);
+        const LoadC nextC(wY, slab + a.slab_offC, ncC, wg, wave, lane);
+        if (DUAL && !SPREAD) nextC.all();
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
         const ColParams cp = col_params<I8>(colp, PH, fc);
-        const float dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1);
+        float dot;
+        if constexpr (SPREAD) dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part, nextC);
+        else dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part);
         TRACE5(2);
         if (finA) pubA[fc] = finish<I8>(dot, cp);
         __syncthreads();
         ++ep;
         if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
         TRACE5(4);
-        if (!DUAL) load_items<PC>(wY, slab + a.slab_offC, ncC, wg, wave, lane);
+        if (!DUAL) nextC.all();
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -862,10 +961,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) {
-          load_items<PD>(wX, slab + a.slab_offD, ncD, wg, wave, lane);
-          if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
-        }
+        const LoadD nextD(wX, slab + a.slab_offD, ncD, wg, wave, lane);
+        if (DUAL && !SPREAD) nextD.all();
+        if (DUAL && !FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         // merge of the slices of each head (flash-decoding): element e of head h is
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
         // derives the weights of its head itself (broadcast LDS reads, no barrier)
@@ -898,7 +996,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         TRACE5(1);
         const ColParams cp = col_params<I8>(colp, PH, fc);
-        const float dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
+        float dot;
+        if constexpr (SPREAD) dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane, nullptr, nullptr, nextD);
+        else dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
         TRACE5(2);
         if (finC) pubC[fc] = own_r + finish<I8>(dot, cp);  // model.js:159
         __syncthreads();
@@ -906,7 +1006,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (tid < ncC) publish(a.bufR1 + wg * PC::CPW + tid, pubC[tid], ep);
         TRACE5(4);
         if (!DUAL) {
-          load_items<PD>(wX, slab + a.slab_offD, ncD, wg, wave, lane);
+          nextD.all();
           if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         }
         TRACE5(5);
@@ -920,16 +1020,19 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) load_e(wY, slab + a.slab_offE);
+        const LoadE nextE(wY, slab + a.slab_offE, ncE, wg, wave, lane);
+        if (DUAL && !SPREAD) nextE.all();
         const ColParams cp = col_params<I8>(colp, PH, fc);
-        const float dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1);
+        float dot;
+        if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, nextE);
+        else dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part);
         TRACE5(2);
         if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
         ++ep;
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
         TRACE5(4);
-        if (!DUAL) load_e(wY, slab + a.slab_offE);
+        if (!DUAL) nextE.all();
         TRACE5(5);
       }
 
@@ -939,35 +1042,41 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // weights of the phase after this one: the next layer's c_attn share with its
         // LayerNorm; after the last layer the final LayerNorm (and, with two register
         // sets, already the first layer's share for the next token)
-        auto request_next = [&]() {
+        auto request_small = [&]() {
           if (li + 1 < a.L) {
-            load_items<PA>(wX, slab + a.slab_stride, ncA, wg, wave, lane);
             request_params(li + 1);
             if (!FOLD) request_ln<D>(lnreg, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
           } else {
             if (!FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
             if (step + 1 < a.nsteps) request_params(0);
-            if (DUAL && step + 1 < a.nsteps) load_items<PA>(wX, slabs, ncA, wg, wave, lane);
           }
         };
+        // (the last layer of the last step requests the first layer's share too and leaves it unused)
+        const LoadA nextA(wX, li + 1 < a.L ? slab + a.slab_stride : slabs, ncA, wg, wave, lane);
         poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL) request_next();
-        const ColParams cpe = col_params<I8>(colp, PH, tid);  // split columns: thread c finishes local column c
-        if constexpr (EKS) gemv_ksplit<PE>(wY, xs1, part, wave, lane);
-        else phase_e<PE, I8>(wY, xs1, part, pubC, pubE, colp, ncE, finE, fc, wave, lane);
+        if (DUAL && !SPREAD && (li + 1 < a.L || step + 1 < a.nsteps)) nextA.all();
+        if (DUAL) request_small();
+        const ColParams cpe = col_params<I8>(colp, PH, tid);  // thread c finishes local column c
+        if constexpr (EKS && SPREAD) gemv_ksplit<PE>(wY, xs1, part, wave, lane, nextA);
+        else if constexpr (EKS) gemv_ksplit<PE>(wY, xs1, part, wave, lane);
+        else if constexpr (SPREAD) gemv_split<PE>(wY, xs1, part, ncE, wave, lane, nextA);
+        else gemv_split<PE>(wY, xs1, part, ncE, wave, lane);
         TRACE5(2);
         __syncthreads();
         ++ep;
         if (tid < ncE) {  // model.js:205
           const float dot = EKS ? column_sum_ksplit<PE>(part, tid) : column_sum<PE>(part, tid);
-          const float r2 = PE::WHOLE ? pubE[tid] : pubC[tid] + finish<I8>(dot, cpe);
+          const float r2 = pubC[tid] + finish<I8>(dot, cpe);
           publish(a.bufR2 + wg * PE::CPW + tid, r2, ep);
         }
         TRACE5(4);
-        if (!DUAL) request_next();
+        if (!DUAL) {
+          request_small();
+          if (li + 1 < a.L) nextA.all();
+        }
         TRACE5(5);
       }
     }
@@ -1109,7 +1218,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     if (a.trace && tid == 0 && step == a.nsteps - 1) a.trace[(size_t)wg * 512 + 501] = __builtin_readcyclecounter();
 #endif
     if (step + 1 < a.nsteps) {
-      if (!DUAL) load_items<PA>(wX, slabs, ncA, wg, wave, lane);
+      if (!DUAL) LoadA(wX, slabs, ncA, wg, wave, lane).all();
       if (!FOLD) request_ln<D>(lnreg, a.lparams + po.ln1g, a.lparams + po.ln1b);
     }
     // ======================= arg-max over the workgroups, finished by everyone =======================
