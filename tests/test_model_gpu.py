@@ -245,13 +245,16 @@ def test_int8_persistent_decode_against_oracle(device):
 
 
 def test_expired_wait_disables_the_persistent_path_and_falls_back(device, monkeypatch):
-    """A bounded wait of the persistent kernel that expires (forced from the host by a poll limit of
-    one round: every workgroup gives up at once and the launch drains normally) is reported as an
-    error, and decoding continues on the per-block kernels with correct results."""
+    """A bounded wait of the persistent kernel that expires (forced from the host: no delay before the
+    first look and no further round after it, so every workgroup gives up at once and the launch
+    drains normally) is reported as an error, and decoding continues on the per-block kernels with
+    correct results."""
     cfg = small_cfg(n_layer=2, n_head=6, n_embd=384, n_ctx=32, vocab_size=90)
-    monkeypatch.setenv("WEBGPT_AMD_SPIN_LIMIT", "1")
+    monkeypatch.setenv("WEBGPT_AMD_SPIN_LIMIT", "0")             # give up at the first look that finds a word missing
+    monkeypatch.setenv("WEBGPT_AMD_POLL_DELAYS", "0,0,0,0,0,0,0")  # and look at once, before any other workgroup can have published
     gpt, tensors = load(cfg, seed=17)
     monkeypatch.delenv("WEBGPT_AMD_SPIN_LIMIT")
+    monkeypatch.delenv("WEBGPT_AMD_POLL_DELAYS")
     w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
     tokens = synth.tokens(17, "prompt", 10, cfg["vocab_size"])
     gpt.prefill(tokens[:8])

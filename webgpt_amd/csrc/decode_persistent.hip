@@ -709,7 +709,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // Input rows alternate between two buffers (xs0: residual stream rows; xs1: merged
   // attention output, MLP hidden row), so that a poll never writes the buffer the
   // dot products of the phase before it may still be reading.
-  extern __shared__ float lds[];
+  // 16-byte aligned behind the static part (676 bytes): a 128-bit LDS access at an address that is not a
+  // multiple of 16 is split by the hardware and takes several times as long
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* xs0 = lds;            // [XS0]
   float* xs1 = xs0 + XS0;      // [XS1]
   float* lnp = xs1 + XS1;      // [2*D] LayerNorm gamma, beta of the next normalising phase

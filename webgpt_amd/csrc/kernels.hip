@@ -842,7 +842,7 @@ __global__ __launch_bounds__(WG) void embed_kernel(const int32_t* __restrict__ i
 constexpr int VOCAB_ROWS_PER_WAVE = 4;
 __global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const float* __restrict__ x,
                                                          const float* __restrict__ wte, float* __restrict__ logits) {
-  extern __shared__ float xs[];
+  extern __shared__ __attribute__((aligned(16))) float xs[];
   for (int c = threadIdx.x; c < (d >> 2); c += WG) st4(xs + 4 * c, ld4(x + 4 * c));
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -875,7 +875,7 @@ __global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const floa
 __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk, float scale, const float* __restrict__ q,
                                                         int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
                                                         size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
-  extern __shared__ float scores[];
+  extern __shared__ __attribute__((aligned(16))) float scores[];
   __shared__ float qs[256];
   __shared__ float red[1024];
   __shared__ float sh[NWAVE];

@@ -300,11 +300,13 @@ static int setup_persistent(Model* m) {
     }
   }
   // a wait that takes this many poll rounds (a quarter of a second) means a workgroup is not running;
-  // WEBGPT_AMD_SPIN_LIMIT lowers it (tests of the fallback force an expiry this way)
+  // WEBGPT_AMD_SPIN_LIMIT lowers it (tests of the fallback force an expiry this way: with 0 a wait
+  // gives up when its first look finds a word missing, which without poll delays is certain)
   a.spin_limit = 1u << 18;
   if (const char* e = getenv("WEBGPT_AMD_SPIN_LIMIT")) {
-    const long v = atol(e);
-    if (v >= 1 && v < (1l << 30)) a.spin_limit = (unsigned)v;
+    char* end = nullptr;
+    const long v = strtol(e, &end, 10);
+    if (end != e && v >= 0 && v < (1l << 30)) a.spin_limit = (unsigned)v;
   }
   a.trace = nullptr;
 #ifdef WGPT_TRACE
