@@ -727,7 +727,11 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
-  if (tid == 0) sh.bail = 0;
+  if (tid == 0) {
+    sh.bail = 0;
+    // a misaligned row buffer would only be slow, not wrong: report it instead of running at a third of the speed
+    if ((reinterpret_cast<size_t>(lds) & 15u) != 0) atomicCAS(a.err, 0, -16);
+  }
   for (int e = tid; e < XS0 + XS1; e += NT) lds[e] = 0.f;  // the padding of xs0 beyond D stays zero for good
 
   // columns this workgroup finishes per phase (fewer than CPW only at the ragged end)

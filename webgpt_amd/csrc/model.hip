@@ -374,6 +374,8 @@ static int check_persistent(Model* m) {
     (void)hipMemset(m->perr, 0, sizeof(int));
     m->persist_ok = false;  // do not trust the exchange buffers again
     m->decode_mode = 0;
+    if (herr == -16)
+      return fail(WGPT_ERR_DEVICE, "persistent decode kernel: its LDS rows are not 16-byte aligned (build problem); the persistent path is now disabled");
     return fail(WGPT_ERR_DEVICE, "persistent decode kernel: a bounded wait expired at epoch %d; the persistent path is now disabled", herr);
   }
   return WGPT_OK;
