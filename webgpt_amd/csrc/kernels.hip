@@ -876,7 +876,7 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
                                                         int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
                                                         size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
   extern __shared__ __attribute__((aligned(16))) float scores[];
-  __shared__ float qs[256];
+  __shared__ __attribute__((aligned(16))) float qs[256];  // read as float4
   __shared__ float red[1024];
   __shared__ float sh[NWAVE];
   const int h = blockIdx.x, i = blockIdx.y;
