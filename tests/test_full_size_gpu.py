@@ -1,4 +1,4 @@
-"""BASELINE configurations at full size. The oracle is too slow to recompute every
+"""The benchmark configurations (GPT-2 117M, 345M, 774M, 1.5B with int8 weights) at full size. The oracle is too slow to recompute every
 step here, so these runs are checked through size-independent properties:
 
   - KV-cache invariance: the logits of the last decode step equal the logits of a
