@@ -55,6 +55,7 @@ struct Model {
   // pinned host words (hipHostMalloc): [0] the token of a single-step call on its way to the device,
   // [1] the error word on its way back, so that a decode call needs one stream synchronisation
   int32_t* pin = nullptr;
+  float* logits_pin = nullptr;  // pinned host copy of the logits of the last call (V floats)
   unsigned epoch = 0;        // last epoch published by earlier launches
 
   hipEvent_t ev0 = nullptr, ev1 = nullptr;

@@ -383,9 +383,12 @@ static int check_persistent(Model* m) {
 
 static int finish_timed(Model* m, float* logits) {
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
-  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+  // the logits cross the bus into pinned memory (a copy into the caller's pageable buffer is staged by the
+  // runtime in pieces) and are handed over with a host copy
+  if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
   if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
+  if (logits) memcpy(logits, m->logits_pin, sizeof(float) * (size_t)m->V);
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   return WGPT_OK;
 }
@@ -393,6 +396,7 @@ static int finish_timed(Model* m, float* logits) {
 static void destroy_model(Model* m) {
   for (void* p : m->allocs) (void)hipFree(p);
   if (m->pin) (void)hipHostFree(m->pin);
+  if (m->logits_pin) (void)hipHostFree(m->logits_pin);
   if (m->ev0) (void)hipEventDestroy(m->ev0);
   if (m->ev1) (void)hipEventDestroy(m->ev1);
   delete m;
@@ -480,6 +484,7 @@ int wgpt_model_finalize(wgpt_model h) {
   if (!m->pin) {
     WGPT_HIP(hipHostMalloc((void**)&m->pin, 2 * sizeof(int32_t), hipHostMallocDefault));
     m->pin[0] = m->pin[1] = 0;
+    WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * (size_t)m->V, hipHostMallocDefault));
   }
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_samp_dev))) return rc;
