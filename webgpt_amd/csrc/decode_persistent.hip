@@ -973,8 +973,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // merge of the slices of each head (flash-decoding): element e of head h is
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
         // derives the weights of its head itself (broadcast LDS reads, no barrier)
-#pragma unroll
-        for (int k = 0; k < (D + NT - 1) / NT; ++k) {
+        constexpr int MERGE_ROUNDS = (D + NT - 1) / NT;
+        static_for<MERGE_ROUNDS>([&](auto KK) {
+          constexpr int k = decltype(KK)::value;
           const int e = tid + k * NT;
           if (k * NT + NT <= D || e < D) {
             const int h = e / HS, c = e - h * HS;
@@ -995,7 +996,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
             }
             xs1[e] = val * fast_rcp(Lsum);
           }
-        }
+          // (the few dot products of this phase cannot take c_fc's requests between them: the rounds of the merge do)
+          if constexpr (SPREAD) {
+            nextD.template slot<k, MERGE_ROUNDS>();
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
         if (XS0 > D) {  // the hidden row of the layer before reached into the padding
           for (int e = D + tid; e < XS0; e += NT) xs1[e] = 0.f;
         }
@@ -1003,8 +1009,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE5(1);
         const ColParams cp = col_params<I8>(colp, PH, fc);
         float dot;
-        if constexpr (SPREAD) dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane, nullptr, nullptr, nextD);
-        else dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
+        dot = gemv_whole<PC, false, false>(wY, xs1, lnp, ncC, wave, lane);
         TRACE5(2);
         if (finC) pubC[fc] = own_r + finish<I8>(dot, cp);  // model.js:159
         __syncthreads();
