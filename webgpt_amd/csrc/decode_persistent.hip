@@ -84,6 +84,25 @@ __device__ __forceinline__ float wave_sum(float v) {
   v = dpp_add<0x143, 0xc>(v);
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
+// N sums side by side, step by step: a step's N instructions are independent, so none waits for the one
+// before it (one sum after the other is six dependent steps each).
+template <int N>
+__device__ __forceinline__ void wave_sum_n(float (&v)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x111, 0xf>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x112, 0xf>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x114, 0xf>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x118, 0xf>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x142, 0xa>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = dpp_add<0x143, 0xc>(v[i]);
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[i]), 63));
+}
 // Sum over each row of 16 lanes, every lane of the row gets it (row rotations).
 __device__ __forceinline__ float row16_sum(float v) {
   v = dpp_add<0x128, 0xf>(v);
@@ -607,11 +626,10 @@ __device__ __forceinline__ void gemv_ksplit(const WS& ws, const float* xs, float
       pin_requests<R>();
     });
   });
+  wave_sum_n(acc);
 #pragma unroll
-  for (int c = 0; c < P::CPW; ++c) {
-    const float r = wave_sum(acc[c]);
-    if (lane == 0) part[c * NW + wave] = r;
-  }
+  for (int c = 0; c < P::CPW; ++c)
+    if (lane == 0) part[c * NW + wave] = acc[c];
 }
 template <class P>
 __device__ __forceinline__ float column_sum_ksplit(const float* part, int c) {
