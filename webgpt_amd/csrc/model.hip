@@ -290,7 +290,7 @@ static int setup_persistent(Model* m) {
     static const int tuned[4][7] = {{20, 0, 28, 96, 28, 24, 32},    // d <= 768
                                     {32, 0, 48, 96, 40, 32, 64},    // d = 1024
                                     {16, 0, 48, 96, 4, 20, 40},     // d = 1280
-                                    {16, 12, 48, 48, 32, 24, 8}};   // d = 1600, int8
+                                    {16, 12, 28, 96, 28, 20, 8}};   // d = 1600, int8
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : 3];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
     if (const char* e = getenv("WEBGPT_AMD_POLL_DELAYS")) {
