@@ -352,10 +352,19 @@ struct ItemLoader {
     static_for<E - B>([&](auto k) { this->template item<B + decltype(k)::value>(); });
   }
   // All of them at once (the code of a run of requests is shorter than that of the same requests one by one).
-  __device__ __forceinline__ void all() const {
+  __device__ __forceinline__ void all() const { part<0, 1>(); }
+  // A compute unit's memory pipeline takes requests for about 32 KB without holding the waves (measured with
+  // all 256 compute units requesting at once: 16 KB 33 clocks, 32 KB 190, 48 KB 540, 64 KB 1330, 96 KB 2500):
+  // a phase whose share is larger is requested in two halves (whole columns, or runs of items), the second
+  // when the phase has published.
+  static constexpr bool HALVES = LAYOUT != LAY_KSPLIT && P::ITEMS * (int)sizeof(T) * 64 > 24 * 1024 &&
+                                 (LAYOUT == LAY_WHOLE ? P::CW >= 2 : P::IPW >= 2);
+  // Part H of NH: of the whole columns of this wave, or of its run of items.
+  template <int H, int NH>
+  __device__ __forceinline__ void part() const {
     if constexpr (LAYOUT == LAY_WHOLE) {
 #pragma unroll
-      for (int cc = 0; cc < P::CW; ++cc) {
+      for (int cc = P::CW * H / NH; cc < P::CW * (H + 1) / NH; ++cc) {
         const int c = wave + cc * NW;
 #pragma unroll
         for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
@@ -369,7 +378,7 @@ struct ItemLoader {
       for_wave(wave, [&](auto W) {
         constexpr int J0 = decltype(W)::value * P::IPW;
 #pragma unroll
-        for (int i = 0; i < P::IPW; ++i) {
+        for (int i = P::IPW * H / NH; i < P::IPW * (H + 1) / NH; ++i) {
           zero_item(ws.w[i]);
           if (J0 + i < P::ITEMS) {
             if (!P::RAGGED || J0 + i < nitems) ws.w[i] = ld_stream(wgbase + (J0 + i) * 64);
@@ -377,8 +386,17 @@ struct ItemLoader {
         }
       });
     } else {
+      static_assert(NH == 1, "the segment layout is requested whole or item by item");
       static_for<N>([&](auto k) { this->template item<decltype(k)::value>(); });
     }
+  }
+  // at the start of the phase before / after that phase has published
+  __device__ __forceinline__ void early() const {
+    if constexpr (HALVES) part<0, 2>();
+    else all();
+  }
+  __device__ __forceinline__ void late() const {
+    if constexpr (HALVES) part<1, 2>();
   }
 };
 
@@ -845,7 +863,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         const LoadC nextC(wY, slab + a.slab_offC, ncC, wg, wave, lane);
-        if (DUAL && !SPREAD) nextC.all();
+        if (DUAL && !SPREAD) nextC.early();
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
         const ColParams cp = col_params<I8>(colp, PH, fc);
         float dot;
@@ -858,6 +876,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
         TRACE5(4);
         if (!DUAL) nextC.all();
+        else if (!SPREAD) nextC.late();
         TRACE5(5);
         if (att_role) {
           // this layer's cached keys and values of the slice
@@ -986,7 +1005,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         const LoadD nextD(wX, slab + a.slab_offD, ncD, wg, wave, lane);
-        if (DUAL && !SPREAD) nextD.all();
+        if (DUAL && !SPREAD) nextD.early();
         if (DUAL && !FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         // merge of the slices of each head (flash-decoding): element e of head h is
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
@@ -1037,7 +1056,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (!DUAL) {
           nextD.all();
           if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
-        }
+        } else if (!SPREAD) nextD.late();
         TRACE5(5);
       }
 
@@ -1050,7 +1069,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         wait_loads();
         TRACE(1 + li * 8 + PH);
         const LoadE nextE(wY, slab + a.slab_offE, ncE, wg, wave, lane);
-        if (DUAL && !SPREAD) nextE.all();
+        if (DUAL && !SPREAD) nextE.early();
         const ColParams cp = col_params<I8>(colp, PH, fc);
         float dot;
         if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, nextE);
@@ -1062,6 +1081,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
         TRACE5(4);
         if (!DUAL) nextE.all();
+        else if (!SPREAD) nextE.late();
         TRACE5(5);
       }
 
@@ -1086,7 +1106,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if (DUAL && !SPREAD && (li + 1 < a.L || step + 1 < a.nsteps)) nextA.all();
+        if (DUAL && !SPREAD && (li + 1 < a.L || step + 1 < a.nsteps)) nextA.early();
         if (DUAL) request_small();
         const ColParams cpe = col_params<I8>(colp, PH, tid);  // thread c finishes local column c
         if constexpr (EKS && SPREAD) gemv_ksplit<PE>(wY, xs1, part, wave, lane, nextA);
@@ -1105,7 +1125,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (!DUAL) {
           request_small();
           if (li + 1 < a.L) nextA.all();
-        }
+        } else if (!SPREAD && (li + 1 < a.L || step + 1 < a.nsteps)) nextA.late();
         TRACE5(5);
       }
     }
