@@ -287,7 +287,7 @@ static int setup_persistent(Model* m) {
     // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
     // curves are flat within a few percent around them and over context length);
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
-    static const int tuned[4][7] = {{20, 0, 28, 96, 28, 24, 32},    // d <= 768
+    static const int tuned[4][7] = {{16, 0, 20, 96, 20, 28, 48},    // d <= 768
                                     {32, 0, 48, 96, 40, 32, 64},    // d = 1024
                                     {16, 0, 48, 96, 4, 20, 40},     // d = 1280
                                     {16, 12, 28, 96, 28, 20, 8}};   // d = 1600, int8
