@@ -136,7 +136,7 @@ def main():
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
     # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)
-    traffic = 520.3e6 if (persistent and args.config == "gpt2-117m") else None
+    traffic = 520.2e6 if (persistent and args.config == "gpt2-117m") else None
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
