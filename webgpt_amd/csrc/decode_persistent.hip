@@ -400,6 +400,22 @@ struct ItemLoader {
   }
 };
 
+// Of a share that is dealt out between dot products, only the first NUM/DEN (the rest is requested when the
+// phase has published: `rest`).
+template <class L, int NUM, int DEN>
+struct Leading {
+  static constexpr int NE = L::N * NUM / DEN;
+  const L& l;
+  template <int J, int NS>
+  __device__ __forceinline__ void slot() const {
+    constexpr int B = J * NE / NS, E = (J + 1) * NE / NS;
+    static_for<E - B>([&](auto k) { l.template item<B + decltype(k)::value>(); });
+  }
+  __device__ __forceinline__ void rest() const {
+    static_for<L::N - NE>([&](auto k) { l.template item<NE + decltype(k)::value>(); });
+  }
+};
+
 // What a dot-product loop calls after item J of its NS when nothing is to be requested.
 struct NoRequests {
   template <int J, int NS>
@@ -735,6 +751,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   typedef typename PS::E PE;
   constexpr int D = C::D, HS = C::HS, H = C::H, HID = C::HID, SPLIT = C::SPLIT, MAXI = PS::MAXI;
   constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS, SPREAD = PS::SPREAD;
+  constexpr int SPN = 2, SPD = 3;  // share of a dealt-out request run that goes between the dot products
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
@@ -1011,6 +1028,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s; every thread
         // derives the weights of its head itself (broadcast LDS reads, no barrier)
         constexpr int MERGE_ROUNDS = (D + NT - 1) / NT;
+        const Leading<LoadD, SPN, SPD> leadD{nextD};
         static_for<MERGE_ROUNDS>([&](auto KK) {
           constexpr int k = decltype(KK)::value;
           const int e = tid + k * NT;
@@ -1035,7 +1053,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
           // (the few dot products of this phase cannot take c_fc's requests between them: the rounds of the merge do)
           if constexpr (SPREAD) {
-            nextD.template slot<k, MERGE_ROUNDS>();
+            leadD.template slot<k, MERGE_ROUNDS>();
             __builtin_amdgcn_sched_barrier(0);
           }
         });
@@ -1057,6 +1075,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           nextD.all();
           if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
         } else if (!SPREAD) nextD.late();
+        else leadD.rest();
         TRACE5(5);
       }
 
@@ -1072,7 +1091,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (DUAL && !SPREAD) nextE.early();
         const ColParams cp = col_params<I8>(colp, PH, fc);
         float dot;
-        if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, nextE);
+        const Leading<LoadE, SPN, SPD> leadE{nextE};
+        if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, leadE);
         else dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part);
         TRACE5(2);
         if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
@@ -1082,6 +1102,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE5(4);
         if (!DUAL) nextE.all();
         else if (!SPREAD) nextE.late();
+        else leadE.rest();
         TRACE5(5);
       }
 
