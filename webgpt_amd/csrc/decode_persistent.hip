@@ -112,6 +112,25 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// v of lane l and of lane l ^ 16 (l ^ 32) as a pair, through the row (half-wave) swap instructions: plain
+// vector instructions, where a shuffle goes through the LDS pipeline.
+__device__ __forceinline__ void pair16(float v, float& a, float& b) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void pair32(float v, float& a, float& b) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_sum(float v) { float a, b; pair16(v, a, b); return a + b; }
+__device__ __forceinline__ float xor32_sum(float v) { float a, b; pair32(v, a, b); return a + b; }
+__device__ __forceinline__ float xor16_max(float v) { float a, b; pair16(v, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float xor32_max(float v) { float a, b; pair32(v, a, b); return fmaxf(a, b); }
+
 // Hardware approximations (about 1 ulp each), used where an exact quotient, square
 // root or exponential would put a dozen dependent instructions on a phase's
 // critical path; the difference is orders of magnitude inside the parity tolerance.
@@ -980,13 +999,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
         }
         // the four groups of a wave combine in registers (rescaled to the wave's maximum) ...
-        float mw = fmaxf(m, __shfl_xor(m, 16));
-        mw = fmaxf(mw, __shfl_xor(mw, 32));
+        float mw = xor16_max(m);
+        mw = xor32_max(mw);
         const float f = m > -INFINITY ? fast_exp(m - mw) : 0.f;
         l *= f;
         o.x *= f; o.y *= f; o.z *= f; o.w *= f;
-        l += __shfl_xor(l, 16); o.x += __shfl_xor(o.x, 16); o.y += __shfl_xor(o.y, 16); o.z += __shfl_xor(o.z, 16); o.w += __shfl_xor(o.w, 16);
-        l += __shfl_xor(l, 32); o.x += __shfl_xor(o.x, 32); o.y += __shfl_xor(o.y, 32); o.z += __shfl_xor(o.z, 32); o.w += __shfl_xor(o.w, 32);
+        l = xor16_sum(l); o.x = xor16_sum(o.x); o.y = xor16_sum(o.y); o.z = xor16_sum(o.z); o.w = xor16_sum(o.w);
+        l = xor32_sum(l); o.x = xor32_sum(o.x); o.y = xor32_sum(o.y); o.z = xor32_sum(o.z); o.w = xor32_sum(o.w);
         // ... and the eight waves through LDS: (o[HS], m, l) per wave
         if (lane < 16) {
           *reinterpret_cast<float4*>(part + wave * (HS + 4) + sub * 4) = o;
