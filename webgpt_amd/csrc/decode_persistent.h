@@ -11,11 +11,12 @@ namespace wgpt {
 
 constexpr int PD_THREADS = 512;  // threads per workgroup
 constexpr int PD_GRID = 256;     // workgroups: one per compute unit of an MI355X
-constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase
+constexpr int PD_SPLIT = 4;      // position slices per head in the attention phase (contexts up to PD_SHORT_KEYS)
+constexpr int PD_SPLIT_LONG = 8; // ... beyond
 constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
 constexpr int PD_COLP = 256;     // floats of one workgroup's column parameters of a layer (4 phases x 32 columns x {bias, scale})
-constexpr int PD_MAXKV = 8;      // key batches (of 32) a slice can hold: n_ctx <= 32*PD_MAXKV*PD_SPLIT
-constexpr int PD_SHORT_KEYS = 32 * (PD_MAXKV / 2) * PD_SPLIT;  // longest context of the instantiation with half the key batches
+constexpr int PD_KVBATCH = 4;    // key batches (of 32) a slice holds in registers: n_ctx <= 32*PD_KVBATCH*PD_SPLIT_LONG
+constexpr int PD_SHORT_KEYS = 32 * PD_KVBATCH * PD_SPLIT;  // longest context of the instantiation with PD_SPLIT slices
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
 // [w*cpw, (w+1)*cpw) of N; a column is S segments ("items") of 256 contraction elements,

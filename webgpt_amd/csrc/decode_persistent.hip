@@ -170,11 +170,12 @@ __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70
 // constant, so the per-phase code is loads, FMAs and a few scalar compares. (A wave
 // retires only one instruction every few cycles; index arithmetic on the critical
 // path of a phase costs as much as the hop between phases.)
-template <int D_, int H_, bool I8_ = false>
+template <int D_, int H_, bool I8_ = false, int SPLIT_ = PD_SPLIT>
 struct Shape {
   static constexpr int D = D_, H = H_, HS = D_ / H_, HID = 4 * D_;
   static constexpr bool I8 = I8_;  // linear weights are int8 (4 contraction elements per 32-bit word) + per-column scale
-  static constexpr int G = PD_GRID, SPLIT = PD_SPLIT;
+  static constexpr int G = PD_GRID, SPLIT = SPLIT_;  // SPLIT: position slices per head in the attention phase
+  static_assert(H * SPLIT <= PD_GRID, "a workgroup per head and slice");
   static constexpr int SD = (D + SEG - 1) / SEG;      // segments of a D-long contraction
   static constexpr int SH = (HID + SEG - 1) / SEG;    // segments of a HID-long contraction
   static constexpr int ATTW = H * SPLIT * (HS + 2);   // words of the attention exchange buffer
@@ -1511,15 +1512,16 @@ hipError_t launch_kv(const PersistentArgs& a, hipStream_t s) {
   return hipGetLastError();
 }
 
-// A launch whose last step sees at most half of the longest context runs the instantiation with half
-// the key/value registers (32 fewer float4 per lane: the shapes at the register limit spill less, the
-// others schedule more freely).
-template <class C>
+// A slice of a head holds at most PD_KVBATCH batches of 32 positions in registers. A launch whose last step
+// sees more than PD_SHORT_KEYS positions runs the instantiation with twice the slices per head: a compute
+// unit streams only ~50 GB/s (32 KB in flight per round trip), and the keys and values of a quarter of a
+// long context take an attention workgroup longer to fetch than everything else it does in the layer.
+template <int D, int H, bool I8>
 hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
   const int keys = a.pos0 + a.nsteps;  // positions the last step attends to
-  if (keys > 32 * PD_MAXKV * PD_SPLIT) return hipErrorInvalidValue;
-  if (keys <= PD_SHORT_KEYS) return launch_kv<C, PD_MAXKV / 2>(a, s);
-  return launch_kv<C, PD_MAXKV>(a, s);
+  if (keys > 32 * PD_KVBATCH * PD_SPLIT_LONG) return hipErrorInvalidValue;
+  if (keys <= PD_SHORT_KEYS) return launch_kv<Shape<D, H, I8, PD_SPLIT>, PD_KVBATCH>(a, s);
+  return launch_kv<Shape<D, H, I8, PD_SPLIT_LONG>, PD_KVBATCH>(a, s);
 }
 
 }  // namespace
@@ -1552,7 +1554,7 @@ hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g,
 }
 
 bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
-  if (((n_ctx + PD_SPLIT - 1) / PD_SPLIT + 31) / 32 > PD_MAXKV) return false;
+  if (n_ctx > 32 * PD_KVBATCH * PD_SPLIT_LONG) return false;
   if (weight_dtype == 1) return d == 1600 && n_head == 25;
   return (d == 384 && n_head == 6) || (d == 768 && n_head == 12) || (d == 1024 && n_head == 16) ||
          (d == 1280 && n_head == 20);
@@ -1567,12 +1569,12 @@ hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype,
 
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
   if (!persistent_supports(a.d, a.H, a.ctx, a.weight_dtype) || a.top_k < 1 || a.top_k > PD_TOPK) return hipErrorInvalidValue;
-  if (a.weight_dtype == 1) return launch_t<Shape<1600, 25, true>>(a, s);
+  if (a.weight_dtype == 1) return launch_t<1600, 25, true>(a, s);
   switch (a.d) {
-    case 384: return launch_t<Shape<384, 6>>(a, s);
-    case 768: return launch_t<Shape<768, 12>>(a, s);
-    case 1024: return launch_t<Shape<1024, 16>>(a, s);
-    case 1280: return launch_t<Shape<1280, 20>>(a, s);
+    case 384: return launch_t<384, 6, false>(a, s);
+    case 768: return launch_t<768, 12, false>(a, s);
+    case 1024: return launch_t<1024, 16, false>(a, s);
+    case 1280: return launch_t<1280, 20, false>(a, s);
   }
   return hipErrorInvalidValue;
 }

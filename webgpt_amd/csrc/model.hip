@@ -202,7 +202,7 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 // m->persist_ok false (and the per-block path in charge) for shapes it does not cover.
 static int setup_persistent(Model* m) {
   m->persist_ok = false;
-  const int d = m->d, hid = 4 * d, G = PD_GRID, split = PD_SPLIT;
+  const int d = m->d, hid = 4 * d, G = PD_GRID, split = PD_SPLIT_LONG;  // (the exchange buffer of the larger split)
   const bool i8 = m->p.weight_dtype == 1;
   if (m->hs != 64) return WGPT_OK;
   if (rt().compute_units < G) return WGPT_OK;
