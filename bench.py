@@ -6,7 +6,7 @@ device-resident KV cache, followed by the on-device arg-max that feeds the next
 step. Weights, KV cache and the first token are resident in HBM when the timed
 region starts; nothing crosses PCIe inside it. Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config gpt2-117m]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config gpt2-117m] [--prompt T]
 """
 import argparse
 import json
@@ -53,6 +53,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="gpt2-117m")
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--prompt", type=int, default=None,
+                    help="prompt length (default: the configuration's); the decode steps that follow must fit n_ctx")
     ap.add_argument("--mode", type=int, default=None, help="decode implementation (default: library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
@@ -69,8 +71,10 @@ def main():
     from webgpt_amd._lib import WgptError
 
     cfg = dict(synth.CONFIGS[args.config])
+    if args.prompt is not None:
+        cfg["prompt"] = args.prompt
     if args.steps is None:
-        args.steps = cfg["decode"] - args.warmup
+        args.steps = min(cfg["decode"], cfg["n_ctx"] - cfg["prompt"]) - args.warmup
     if args.steps < 1 or cfg["prompt"] + args.warmup + args.steps > cfg["n_ctx"]:
         print(f"bench.py: prompt {cfg['prompt']} + warmup + steps exceeds n_ctx {cfg['n_ctx']}", file=sys.stderr)
         sys.exit(2)
@@ -93,10 +97,12 @@ def main():
 
     # prefill (untimed for the headline; reported separately)
     gpt.prefill(prompt)  # first call also loads the code objects
-    t0 = time.perf_counter()
-    logits = gpt.prefill(prompt)
-    prefill_wall_ms = (time.perf_counter() - t0) * 1000.0
-    prefill_gpu_ms = gpt.lastGpuMs
+    runs = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        logits = gpt.prefill(prompt)
+        runs.append(((time.perf_counter() - t0) * 1000.0, gpt.lastGpuMs))
+    prefill_wall_ms, prefill_gpu_ms = float(np.median([r[0] for r in runs])), float(np.median([r[1] for r in runs]))
     tok = int(np.argmax(logits))
     T, L, d = len(prompt), cfg["n_layer"], cfg["n_embd"]
     prefill_flops = 2.0 * T * 12 * L * d * d + 2.0 * L * T * T * d
@@ -136,7 +142,7 @@ def main():
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
     # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)
-    traffic = 520.2e6 if (persistent and args.config == "gpt2-117m") else None
+    traffic = 520.2e6 if (persistent and args.config == "gpt2-117m" and args.prompt is None) else None
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
@@ -157,7 +163,7 @@ def main():
         "tokens_per_s": round(1000.0 / ms_per_step, 1),
         "gpu_ms_per_token": round(gpu_ms / args.steps, 5),
         "prefill_tokens_per_s": round(len(prompt) / (prefill_gpu_ms * 1e-3), 1),
-        "prefill_ms": round(prefill_gpu_ms, 3),
+        "prefill_ms": round(prefill_gpu_ms, 3),  # HIP-event time, median of 5 calls after one untimed
         "prefill_wall_ms": round(prefill_wall_ms, 3),
         # whole prefill (all kernels) against the fp32 MFMA peak: linear-layer flops 2*T*12*L*d^2 + causal attention 2*L*T^2*d
         "prefill_tflops": round(prefill_flops / (prefill_gpu_ms * 1e-3) / 1e12, 2),
