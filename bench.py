@@ -141,8 +141,10 @@ def main():
             persistent = False
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
-    # measured with rocprofv3 --pmc on single-token launches at context 186 (profiles/decode_persistent_gpt2-117m.md)
-    traffic = 520.2e6 if (persistent and args.config == "gpt2-117m" and args.prompt is None) else None
+    # measured with rocprofv3 --pmc on single-token launches of the host loop that follows 40 timed steps, i.e. at
+    # contexts 171..202 (117M, int8), 555..586 (345M), 107..138 (774M); profiles/decode_persistent_*.md
+    measured = {"gpt2-117m": 520.2e6, "gpt2-345m": 1564.7e6, "gpt2-774m": 3187.3e6, "gpt2-1.5b-int8": 2209.7e6}
+    traffic = measured.get(args.config) if (persistent and args.prompt is None) else None
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
