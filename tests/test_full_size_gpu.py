@@ -1,4 +1,4 @@
-"""The benchmark configurations (GPT-2 117M, 345M, 774M, 1.5B with int8 weights) at full size. The oracle is too slow to recompute every
+"""The benchmark configurations (GPT-2 117M, 345M, 774M, 1.5B with int8 weights) and the fp32 1.5B shape at full size. The oracle is too slow to recompute every
 step here, so these runs are checked through size-independent properties:
 
   - KV-cache invariance: the logits of the last decode step equal the logits of a
@@ -76,3 +76,8 @@ def test_gpt2_774m_to_full_context():
 
 def test_gpt2_1p5b_int8_full():
     run_config("gpt2-1.5b-int8", 128, 64)
+
+
+def test_gpt2_1p5b_fp32_across_512_positions():
+    # the fourth model the reference offers (index.html:31); both instantiations of the persistent kernel
+    run_config("gpt2-1.5b", 490, 40)

@@ -1557,7 +1557,7 @@ bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
   if (n_ctx > 32 * PD_KVBATCH * PD_SPLIT_LONG) return false;
   if (weight_dtype == 1) return d == 1600 && n_head == 25;
   return (d == 384 && n_head == 6) || (d == 768 && n_head == 12) || (d == 1024 && n_head == 16) ||
-         (d == 1280 && n_head == 20);
+         (d == 1280 && n_head == 20) || (d == 1600 && n_head == 25);
 }
 
 hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype, float* out, hipStream_t s) {
@@ -1575,6 +1575,7 @@ hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
     case 768: return launch_t<768, 12, false>(a, s);
     case 1024: return launch_t<1024, 16, false>(a, s);
     case 1280: return launch_t<1280, 20, false>(a, s);
+    case 1600: return launch_t<1600, 25, false>(a, s);
   }
   return hipErrorInvalidValue;
 }

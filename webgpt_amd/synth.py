@@ -19,6 +19,7 @@ CONFIGS = {
     "gpt2-117m": dict(n_layer=12, n_head=12, n_embd=768, n_ctx=1024, vocab_size=50257, prompt=128, decode=256, dtype="f32"),
     "gpt2-345m": dict(n_layer=24, n_head=16, n_embd=1024, n_ctx=1024, vocab_size=50257, prompt=512, decode=512, dtype="f32"),
     "gpt2-774m": dict(n_layer=36, n_head=20, n_embd=1280, n_ctx=1024, vocab_size=50257, prompt=64, decode=960, dtype="f32"),
+    "gpt2-1.5b": dict(n_layer=48, n_head=25, n_embd=1600, n_ctx=1024, vocab_size=50257, prompt=128, decode=256, dtype="f32"),
     "gpt2-1.5b-int8": dict(n_layer=48, n_head=25, n_embd=1600, n_ctx=1024, vocab_size=50257, prompt=128, decode=256, dtype="int8"),
 }
 
