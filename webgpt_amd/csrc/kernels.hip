@@ -152,6 +152,47 @@ __global__ __launch_bounds__(WG) void gemv_reduce(int M, int N, int S, const flo
   }
 }
 
+// gemv_reduce for the many slices of a matrix-vector product (S = K / 64): sixteen threads share an output
+// float4, thread ty summing slices ty, ty + 16, ... (loads in flight together instead of S in a row), the
+// sixteen sums combined in ascending ty by the first of them. Same result for every run; bias last.
+__global__ __launch_bounds__(WG) void gemv_reduce_wide(int M, int N, int S, const float* __restrict__ part,
+                                                        const float* __restrict__ bias, float* C, int ldc, int epi,
+                                                        const float* resid) {
+  __shared__ float4 red[16][16];
+  const int n4 = N >> 2;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int idx = blockIdx.x * 16 + tx;
+  const bool live = idx < M * n4;
+  const int r = live ? idx / n4 : 0, n0 = live ? (idx - r * n4) * 4 : 0;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (live) {
+#pragma unroll 4
+    for (int sp = ty; sp < S; sp += 16) {
+      const float4 v = ld4(part + ((size_t)sp * M + r) * N + n0);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+  }
+  red[ty][tx] = s;
+  __syncthreads();
+  if (ty != 0 || !live) return;
+#pragma unroll
+  for (int j = 1; j < 16; ++j) {
+    const float4 v = red[j][tx];
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (bias) {
+    const float4 b = ld4(bias + n0);
+    s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+  }
+  if (epi == EPI_GELU) {
+    s.x = gelu_ref(s.x); s.y = gelu_ref(s.y); s.z = gelu_ref(s.z); s.w = gelu_ref(s.w);
+  } else if (epi == EPI_RESIDUAL) {
+    const float4 q = ld4(resid + (size_t)r * ldc + n0);
+    s.x += q.x; s.y += q.y; s.z += q.z; s.w += q.w;
+  }
+  st4(C + (size_t)r * ldc + n0, s);
+}
+
 // gemv_reduce of one row followed by the LayerNorm of that row (layernorm_kernel's arithmetic and order of
 // operations, thread t holding the float4 t, t + WG, ... of the row): C gets the finished row, ln_out its
 // normalisation. One workgroup per row; N a multiple of 4, at most 4 * WG * REDUCE_LN_MAXV.
@@ -1382,6 +1423,13 @@ inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 }  // namespace
 
+// second pass of a matrix-vector product: slices side by side once there are sixteen of them
+static void launch_gemv_reduce(int M, int N, int S, const float* workspace, const float* bias, float* C, int ldc, int epi,
+                               const float* resid, hipStream_t s) {
+  if (S >= 16) gemv_reduce_wide<<<cdiv((size_t)M * (N >> 2), 16), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  else gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+}
+
 size_t gemv_workspace_floats(int M, int N, int K) {
   return (size_t)cdiv(K, GEMV_KCHUNK) * (size_t)(M < 1 ? 1 : M) * (size_t)N;
 }
@@ -1397,7 +1445,7 @@ hipError_t launch_gemv_kn(int M, int N, int K, const float* A, int lda, const fl
     case 4: gemv_kn_partial<4><<<grid, WG, 0, s>>>(N, K, A, lda, W, ldw, workspace); break;
     default: return hipErrorInvalidValue;
   }
-  gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  launch_gemv_reduce(M, N, S, workspace, bias, C, ldc, epi, resid, s);
   return hipGetLastError();
 }
 
@@ -1413,7 +1461,7 @@ hipError_t launch_gemv_kn_i8(int M, int N, int K, const float* A, int lda, const
     case 4: gemv_kn_i8_partial<4><<<grid, WG, 0, s>>>(N, K, A, lda, Wq, ldwq, scale, workspace); break;
     default: return hipErrorInvalidValue;
   }
-  gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  launch_gemv_reduce(M, N, S, workspace, bias, C, ldc, epi, resid, s);
   return hipGetLastError();
 }
 
