@@ -81,3 +81,19 @@ def test_gpt2_1p5b_int8_full():
 def test_gpt2_1p5b_fp32_across_512_positions():
     # the fourth model the reference offers (index.html:31); both instantiations of the persistent kernel
     run_config("gpt2-1.5b", 490, 40)
+
+
+def test_gpt2_1p5b_fp32_sampled_tokens_same_in_both_decode_modes():
+    cfg = dict(synth.CONFIGS["gpt2-1.5b"])
+    gpt = GPT(None, "bpe", tensors=dict(synth.make_tensors(cfg, 1)), params=synth.model_params(cfg))
+    gpt.initialize()
+    prompt = [int(t) for t in synth.make_prompt(cfg, 1, 500)]
+    u = np.random.default_rng(5).random(24)
+    drawn = {}
+    for mode in (0, 1):
+        gpt.set_decode_mode(mode)
+        first = int(np.argmax(gpt.prefill(prompt)))
+        drawn[mode] = [int(t) for t in gpt.decode_sample(first, len(u), 5, 0.8, u)]   # positions 500..523
+    assert drawn[0] == drawn[1]
+    assert len(set(drawn[1])) > 1
+    gpt.unloadBuffers()
