@@ -930,15 +930,22 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   const float4 qv = act ? ld4(qs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
   const float* kbase = Kc + h * hstride + sub * 4;
   const float* vbase = Vc + h * hstride + sub * 4;
-  for (int j0 = 0; j0 < nkeys; j0 += ngrp) {
-    const int j = j0 + grp;
-    float part = 0.f;
-    if (act && j < nkeys) {
-      const float4 kv = ld4(kbase + (size_t)j * ldkv);
-      part = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
+  // four key rows per lane group requested before the first is used: one after the other, the ~24 rounds of a
+  // 380-key context each waited a full memory round trip
+  for (int j0 = 0; j0 < nkeys; j0 += 4 * ngrp) {
+    float4 kv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ngrp + grp;
+      kv[u] = (act && j < nkeys) ? ld4(kbase + (size_t)j * ldkv) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
-    if (sub == 0 && j < nkeys) scores[j] = part * scale;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ngrp + grp;
+      float part = (qv.x * kv[u].x + qv.y * kv[u].y) + (qv.z * kv[u].z + qv.w * kv[u].w);
+      for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
+      if (sub == 0 && j < nkeys) scores[j] = part * scale;
+    }
   }
   __syncthreads();
   float m = -3.402823e+38f;
@@ -955,7 +962,15 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   __syncthreads();
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   if (act) {
-    for (int j = grp; j < nkeys; j += ngrp) fma4(acc, scores[j], ld4(vbase + (size_t)j * ldkv));
+    int j = grp;
+    for (; j + 3 * ngrp < nkeys; j += 4 * ngrp) {
+      float4 vv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) vv[u] = ld4(vbase + (size_t)(j + u * ngrp) * ldkv);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) fma4(acc, scores[j + u * ngrp], vv[u]);
+    }
+    for (; j < nkeys; j += ngrp) fma4(acc, scores[j], ld4(vbase + (size_t)j * ldkv));
     st4(red + grp * hs + sub * 4, acc);
   }
   __syncthreads();
@@ -1423,10 +1438,10 @@ inline unsigned cdiv(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 }  // namespace
 
-// second pass of a matrix-vector product: slices side by side once there are sixteen of them
+// second pass of a matrix-vector product: slices side by side (up to sixteen slices the sum is still in ascending order)
 static void launch_gemv_reduce(int M, int N, int S, const float* workspace, const float* bias, float* C, int ldc, int epi,
                                const float* resid, hipStream_t s) {
-  if (S >= 16) gemv_reduce_wide<<<cdiv((size_t)M * (N >> 2), 16), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
+  if (S >= 4) gemv_reduce_wide<<<cdiv((size_t)M * (N >> 2), 16), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
   else gemv_reduce<<<cdiv((size_t)M * (N >> 2), WG), WG, 0, s>>>(M, N, S, workspace, bias, C, ldc, epi, resid);
 }
 
