@@ -1,5 +1,7 @@
 """Parity of the whole-model path (wgpt_prefill / wgpt_decode / wgpt_decode_greedy,
 called through the C ABI) against the CPU oracle's GPT.run restatement."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -266,4 +268,38 @@ def test_expired_wait_disables_the_persistent_path_and_falls_back(device, monkey
     assert close(got, ref.forward(p, w, tokens[:9])), worst(got, ref.forward(p, w, tokens[:9]))
     got = gpt.decode(int(tokens[9]))
     assert close(got, ref.forward(p, w, tokens[:10]))
+    gpt.unloadBuffers()
+
+
+@pytest.mark.parametrize("top_k", [3, 12])
+def test_expired_wait_in_decode_sample_leaves_the_position_unchanged(device, monkeypatch, top_k):
+    """The same host-forced expiry (every kernel exits normally) met by wgpt_decode_sample, on its in-kernel
+    selection (top_k <= 8) and on its one-launch-per-token loop: the call fails, the cache position is what it
+    was before the call, and a retry of the same tokens, now on the per-block kernels, gives the oracle's result."""
+    cfg = small_cfg(n_layer=2, n_head=6, n_embd=384, n_ctx=32, vocab_size=90)
+    monkeypatch.setenv("WEBGPT_AMD_SPIN_LIMIT", "0")
+    monkeypatch.setenv("WEBGPT_AMD_POLL_DELAYS", "0,0,0,0,0,0,0")
+    gpt, tensors = load(cfg, seed=19)
+    monkeypatch.delenv("WEBGPT_AMD_SPIN_LIMIT")
+    monkeypatch.delenv("WEBGPT_AMD_POLL_DELAYS")
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(19, "prompt", 9, cfg["vocab_size"])
+    gpt.prefill(tokens[:8])
+    u = np.array([0.3, 0.6, 0.9])
+    with pytest.raises(WgptError, match="bounded wait expired"):
+        gpt.decode_sample(int(tokens[8]), 3, top_k, 0.8, u)
+    pos = C.c_int(-1)
+    _lib.call("wgpt_model_position", gpt._handle, C.byref(pos))
+    assert pos.value == 8
+    assert gpt._history == [int(t) for t in tokens[:8]]
+    # retry: same token, same draws, per-block kernels; the oracle's loop (model.js:81-85) over full forwards
+    got = [int(t) for t in gpt.decode_sample(int(tokens[8]), 3, top_k, 0.8, u)]
+    hist = [int(t) for t in tokens[:9]]
+    for i in range(3):
+        lg = ref.forward(p, w, np.array(hist, np.int32))
+        nxt, _, _ = ref.sample_topk(lg, top_k, 0.8, float(u[i]))
+        assert got[i] == nxt, (i, got, nxt)
+        hist.append(nxt)
+    _lib.call("wgpt_model_position", gpt._handle, C.byref(pos))
+    assert pos.value == 11
     gpt.unloadBuffers()

@@ -611,18 +611,28 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   const int k = top_k < m->V ? top_k : m->V;
   // up to PD_TOPK candidates the persistent kernel selects and samples itself, all steps in one launch
   const bool in_kernel = persistent && k <= PD_TOPK;
+  // The cache position is committed only when the whole call has succeeded (as wgpt_decode and
+  // wgpt_decode_greedy do): after a failure the caller's history is unchanged, so a retry must find the
+  // model where the call started. A step of the loop below reads m->pos; it is restored on every error path.
+  const int pos_before = m->pos;
+  int rc = WGPT_OK;
   if (in_kernel) {
-    int rc = decode_persistent(m, steps, k, temperature, m->u_dev);
-    if (rc) return rc;
-    m->pos += steps;
+    rc = decode_persistent(m, steps, k, temperature, m->u_dev);
   } else {
-    for (int i = 0; i < steps; ++i) {
+    for (int i = 0; i < steps && rc == WGPT_OK; ++i) {
       // one token per launch: the sampled id in tok_dev[0] is the next launch's input
-      int rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
-      if (rc) return rc;
-      LAUNCH(launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream));
+      rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+      if (rc == WGPT_OK) {
+        hipError_t e = launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream);
+        if (e != hipSuccess) rc = fail(WGPT_ERR_HIP, "launch_sample_topk: %s", hipGetErrorString(e));
+      }
       m->pos += 1;
     }
+  }
+  m->pos = pos_before;
+  if (rc) {
+    (void)hipStreamSynchronize(rt().stream);
+    return rc;
   }
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   WGPT_HIP(hipMemcpyAsync(out_tokens, in_kernel ? m->out_tok_dev : m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
@@ -630,10 +640,8 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
-  if (persistent) {
-    int rc = check_persistent(m);
-    if (rc) return rc;
-  }
+  if (persistent && (rc = check_persistent(m))) return rc;
+  m->pos = pos_before + steps;
   return WGPT_OK;
 }
 
