@@ -15,7 +15,7 @@ from oracle import ref
 from webgpt_amd import synth
 from webgpt_amd.model import GPT
 
-from helpers import close, oracle_weights, worst
+from helpers import close, make_model, oracle_weights, worst
 
 pytestmark = pytest.mark.gpu
 
@@ -67,20 +67,59 @@ def test_gpt2_117m_full():
 
 
 def test_gpt2_345m_full():
-    run_config("gpt2-345m", 512, 511)          # fills the context of 1024 exactly
+    run_config("gpt2-345m", 512, 511, oracle_at=(16,))          # fills the context of 1024 exactly
 
 
 def test_gpt2_774m_to_full_context():
-    run_config("gpt2-774m", 64, 959)           # decode up to the last position of the context
+    run_config("gpt2-774m", 64, 959, oracle_at=(16,))           # decode up to the last position of the context
 
 
 def test_gpt2_1p5b_int8_full():
-    run_config("gpt2-1.5b-int8", 128, 64)
+    run_config("gpt2-1.5b-int8", 128, 255, oracle_at=(16,))     # the configuration's 256 decode tokens
 
 
 def test_gpt2_1p5b_fp32_across_512_positions():
     # the fourth model the reference offers (index.html:31); both instantiations of the persistent kernel
-    run_config("gpt2-1.5b", 490, 40)
+    run_config("gpt2-1.5b", 490, 40, oracle_at=(16,))
+
+
+@pytest.mark.parametrize("name", ["gpt2-117m", "gpt2-345m", "gpt2-774m", "gpt2-1.5b-int8", "gpt2-1.5b"])
+def test_full_depth_decode_step_against_oracle(name):
+    """Every layer of the configuration, LayerNorm gains and biases drawn at random (so the fold of gamma and
+    beta into the decode slabs is not the identity): a prefill, then cached decode steps on both decode paths,
+    each against the oracle's full forward over the same tokens (model.js:104-241). Rounding error grows with
+    depth; this is where the hardware reciprocal / rsqrt / exp2 of the persistent kernel and the int8 kernel's
+    factored column scale would show if they left the tolerance."""
+    cfg = dict(synth.CONFIGS[name])
+    tensors = make_model(cfg, 21, random_ln=True)
+    params = synth.model_params(cfg)
+    params["max_prefill"] = 32
+    gpt = GPT(None, "bpe", tensors=tensors, params=params)
+    gpt.initialize()
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(22, "prompt", 17, cfg["vocab_size"])
+    want = {T: ref.forward(p, w, tokens[:T]) for T in (12, 13, 17)}
+    got = gpt.prefill(tokens[:12])
+    report = {"prefill": worst(got, want[12])}
+    assert close(got, want[12]), (name, "prefill", report)
+    out = {}
+    for mode in (1, 0):
+        gpt.set_decode_mode(mode)
+        gpt.prefill(tokens[:12])
+        out[mode] = [gpt.decode(int(tokens[12 + i])) for i in range(5)]       # positions 12..16
+        for i, T in ((0, 13), (4, 17)):
+            report[f"mode{mode}@{T}"] = worst(out[mode][i], want[T])
+    print(f"\nfull-depth parity {name}: worst |err| / (1e-5 + 1e-4 |want|) = " +
+          ", ".join(f"{k} {v:.3f}" for k, v in report.items()))
+    for mode in (1, 0):
+        for i, T in ((0, 13), (4, 17)):
+            assert close(out[mode][i], want[T]), (name, mode, T, report)
+            assert greedy_ok(out[mode][i], want[T])
+        # the persistent kernel against the per-block kernels directly (for int8: the factored column scale
+        # against the per-weight dequantisation of other/int8-gemm.js:126-132)
+    for i in range(5):
+        assert close(out[1][i], out[0][i]), (name, i, worst(out[1][i], out[0][i]))
+    gpt.unloadBuffers()
 
 
 def test_gpt2_1p5b_fp32_sampled_tokens_same_in_both_decode_modes():
