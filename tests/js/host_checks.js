@@ -18,7 +18,19 @@ const out = {
   transpose: Array.from(w.transpose(new Float32Array([1, 2, 3, 4, 5, 6]), 2, 3)),
   wgSize: [w.wgSize(65, 32), w.wgSize(64, 32)],
   errors: {},
+  gptMethods: Object.getOwnPropertyNames(w.GPT.prototype).sort(),
 };
+// quantizeMatrix / dequantizeMatrix (other/int8-gemm.js:25-62) on a seeded matrix and on the rounding probes
+{
+  const K = 24, N = 8;
+  const m = s.normal(9, "quantize.probe", K * N);
+  m[5] = 0; m[N + 2] = -m[2];
+  for (let k = 0; k < K; k++) m[k * N + 7] = 0;  // an all-zero column
+  const q = w.quantizeMatrix(m, K, N);
+  out.quant = { words: Array.from(q.quantizedMatrix), scale: Array.from(q.scale), dequant: Array.from(w.dequantizeMatrix(q.quantizedMatrix, q.scale, K, N)) };
+  const probe = new Float32Array([-0.5 / 127, 0.5 / 127, -1.5 / 127, 1.0, 2.5 / 127, -2.5 / 127, -1.0, 0.0]);
+  out.quantProbe = Array.from(w.quantizeMatrix(probe, 1, 8, 1.0).quantizedMatrix);
+}
 const dev = { limits: { maxStorageBufferBindingSize: 1 << 20 } };
 w.initializeOperations(dev);
 const tryErr = (name, f) => { try { f(); out.errors[name] = null; } catch (e) { out.errors[name] = e.message; } };

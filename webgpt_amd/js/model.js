@@ -15,6 +15,7 @@ const native = require("./native.js");
 const { Device, initTensor, runPasses } = require("./instructions.js");
 const G = require("./globals.js");
 const { GPT2Tokenizer, SimpleTokenizer } = require("./tokenizer.js");
+const { quantizeMatrix } = require("./quantize.js");
 
 class GPT {
   constructor(folder, type, options = {}) {
@@ -36,6 +37,7 @@ class GPT {
     this._paramsIn = options.params;
     this._flags = options.flags || 0;
     this._tokenization = options.tokenization;
+    this._quantize = options.quantize;  // "int8": quantise the fp32 linear weights while loading (quantize.js)
     this._history = [];
     this.lastGpuMs = 0;
   }
@@ -206,18 +208,34 @@ class GPT {
     };
   }
 
+  // loadModel and the loaders it calls keep the reference's names, order and return shapes
+  // (model.js:270-488). A "buffer" they return is a descriptor { name, dims } of a tensor that
+  // now lives in the library's model (wgpt_model_set_tensor copies the data in); the Q/K/V
+  // entries are column ranges of the fused c_attn, which the library keeps whole.
   async loadModel(folder) {
     if (this.initialized) return console.error("Model already loaded");
-    const params = await this.loadParameters(folder);
-    const names = this._tensors ? Object.keys(this._tensors) : this.directoryNames(params);
-    const int8 = names.some((n) => n.endsWith(".weight.q"));
-    const handle = native.modelCreate(params.n_layer, params.n_head, params.n_embd, params.n_ctx, params.vocab_size, int8 ? 1 : 0, params.max_prefill || 0, this._flags);
-    for (const name of names) {
-      const data = this._tensors ? this._tensors[name] : this.readTensor(folder, name, params);
-      native.modelSetTensor(handle, name, data);
+    const weightsFolder = folder;
+    const params = await this.loadParameters(weightsFolder);
+    const names = this._tensors ? Object.keys(this._tensors) : undefined;
+    const packed = !!names && names.some((n) => n.endsWith(".weight.q"));
+    this._quantise = !packed && (this._quantize || params.quantize) === "int8";
+    const handle = native.modelCreate(params.n_layer, params.n_head, params.n_embd, params.n_ctx, params.vocab_size, packed || this._quantise ? 1 : 0, params.max_prefill || 0, this._flags);
+    this._loading = { handle, params, packed };
+    let output;
+    try {
+      const { embeddingsBuffers, deEmbeddingsBuffers } = await this.loadEmbeddings(params, weightsFolder);
+      const { posEmbdBuffer } = await this.loadPositionalEmbeddings(params, weightsFolder);
+      const layer_buffers = await this.loadLayers(params, weightsFolder);
+      const { normGammaBuffer, normBetaBuffer } = await this.loadFinalLayerNorm(params, weightsFolder);
+      native.modelFinalize(handle);
+      output = { handle, layer_buffers, embeddingsBuffers, deEmbeddingsBuffers, posEmbdBuffer, normGammaBuffer, normBetaBuffer };
+    } catch (e) {
+      native.modelDestroy(handle);
+      throw e;
+    } finally {
+      this._loading = undefined;
     }
-    native.modelFinalize(handle);
-    return [{ handle }, params];
+    return [output, params];
   }
 
   async loadParameters(weightsFolder) {
@@ -233,7 +251,96 @@ class GPT {
     params.hidden_size = params.n_embd * 4;
     params.attention_scale = 1 / Math.sqrt(params.n_embd / params.n_head);
     params.bias = params.bias == undefined ? true : params.bias;
+    // model.js:325-332: the soft limits, against this device's largest buffer (all of HBM)
+    const maxBufferSize = (this.device ? this.device.limits.maxStorageBufferBindingSize : Infinity) / 4;
+    if (params.n_embd * params.n_ctx > maxBufferSize) console.warn("Model load failed: n_embd * n_ctx must be less than maxStorageBufferBindingSize.");
+    if (params.n_embd * params.hidden_size > maxBufferSize) console.warn("Model load failed: n_embd * hidden_size must be less than maxStorageBufferBindingSize.");
+    if (params.n_ctx * params.n_ctx * params.n_head > maxBufferSize) console.warn("Model load failed: n_ctx * n_ctx must be less than maxStorageBufferBindingSize.");
+    if (params.n_embd * params.n_embd * 3 > maxBufferSize) console.warn("Model load failed: n_embd * n_embd * 3 must be less than maxStorageBufferBindingSize.");
     return params;
+  }
+
+  // model.js:339-367. One table serves the gather and the vocabulary projection (row-major wte has
+  // the contraction index contiguous), so both lists hold the same single descriptor.
+  async loadEmbeddings(params, weightsFolder) {
+    const wte = await this.fetchAndInitTensor(`${weightsFolder}/transformer.wte.weight_gpt.bin`, [params.vocab_size, params.n_embd], ["copy_from"]);
+    return { embeddingsBuffers: [wte], deEmbeddingsBuffers: [wte] };
+  }
+
+  async loadPositionalEmbeddings(params, weightsFolder) {
+    const posEmbdBuffer = await this.fetchAndInitTensor(`${weightsFolder}/transformer.wpe.weight_gpt.bin`, [params.n_ctx, params.n_embd], ["copy_from"]);
+    return { posEmbdBuffer };
+  }
+
+  async loadFinalLayerNorm(params, weightsFolder) {
+    const prefix = `${weightsFolder}/transformer.ln_f.`;
+    const [normGammaBuffer, normBetaBuffer] = await Promise.all([
+      this.fetchAndInitTensor(`${prefix}weight_gpt.bin`, [params.n_embd], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}bias_gpt.bin`, [params.n_embd], ["storage"]),
+    ]);
+    return { normGammaBuffer, normBetaBuffer };
+  }
+
+  async loadLayers(params, weightsFolder) {
+    const layerPromises = [];
+    for (let i = 0; i < params.n_layer; i++) layerPromises.push(this.loadLayer(params, weightsFolder, i));
+    return await Promise.all(layerPromises);
+  }
+
+  async loadLayer(params, weightsFolder, layerIndex) {
+    const prefix = `${weightsFolder}/transformer.h.${layerIndex}.`;
+    const d = params.n_embd, hid = params.hidden_size;
+    const [normAttentionGammaBuffer, normAttentionBetaBuffer, qkvWeightArray, qkvBiasArray, linearWeightsBuffer, linearBiasBuffer,
+      normLinearGammaBuffer, normLinearBetaBuffer, firstLayerWeightsBuffer, firstLayerBiasBuffer, secondLayerWeightsBuffer, secondLayerBiasBuffer] = await Promise.all([
+      this.fetchAndInitTensor(`${prefix}ln_1.weight_gpt.bin`, [d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}ln_1.bias_gpt.bin`, [d], ["storage"]),
+      this.fetchAndSplitQKVWeightTensors(`${prefix}attn.c_attn.weight_gpt.bin`, [d, 3 * d], ["storage"]),
+      this.fetchAndSplitQKVBiasTensors(`${prefix}attn.c_attn.bias_gpt.bin`, [d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}attn.c_proj.weight_gpt.bin`, [d, d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}attn.c_proj.bias_gpt.bin`, [d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}ln_2.weight_gpt.bin`, [d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}ln_2.bias_gpt.bin`, [d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}mlp.c_fc.weight_gpt.bin`, [d, hid], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}mlp.c_fc.bias_gpt.bin`, [hid], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}mlp.c_proj.weight_gpt.bin`, [hid, d], ["storage"]),
+      this.fetchAndInitTensor(`${prefix}mlp.c_proj.bias_gpt.bin`, [d], ["storage"]),
+    ]);
+    return { normAttentionGammaBuffer, normAttentionBetaBuffer, qkvWeightArray, qkvBiasArray, linearWeightsBuffer, linearBiasBuffer,
+      normLinearGammaBuffer, normLinearBetaBuffer, firstLayerWeightsBuffer, firstLayerBiasBuffer, secondLayerWeightsBuffer, secondLayerBiasBuffer };
+  }
+
+  // model.js:456-482: the reference cuts c_attn [d, 3d] into three [d, d] matrices (and its bias into
+  // three vectors) on the host. Here the fused tensor goes to the library as it is and Q, K, V are
+  // its column ranges 0..d, d..2d, 2d..3d, which is what the three descriptors say.
+  async fetchAndSplitQKVWeightTensors(url, dims, ops) {
+    const fused = await this.fetchAndInitTensor(url, [dims[0], 3 * dims[0]], ops);
+    return [0, 1, 2].map((part) => ({ name: fused.name, dims: [dims[0], dims[0]], columns: [part * dims[0], (part + 1) * dims[0]] }));
+  }
+
+  async fetchAndSplitQKVBiasTensors(url, dims, ops) {
+    const fused = await this.fetchAndInitTensor(url, [3 * dims[0]], ops);
+    return [0, 1, 2].map((part) => ({ name: fused.name, dims: [dims[0]], columns: [part * dims[0], (part + 1) * dims[0]] }));
+  }
+
+  // model.js:484-488: reads <name>_gpt.bin (or the in-memory tensor of that name) and hands it to the
+  // model being loaded. A linear weight goes in as it is, as its packed int8 words and column scales
+  // when the directory holds those, or quantised here when the model was opened with quantize: "int8".
+  async fetchAndInitTensor(url, dims, ops) {
+    const { handle, params, packed } = this._loading;
+    const name = path.basename(url).replace(/_gpt\.bin$/, "");
+    const linear = /^transformer\.h\.\d+\.(attn\.c_attn|attn\.c_proj|mlp\.c_fc|mlp\.c_proj)\.weight$/.test(name);
+    const fetch = (n) => (this._tensors ? this._tensors[n] : this.readTensor(path.dirname(url), n, params));
+    if (linear && packed) {
+      native.modelSetTensor(handle, name + ".q", fetch(name + ".q"));
+      native.modelSetTensor(handle, name + ".scale", fetch(name + ".scale"));
+    } else if (linear && this._quantise) {
+      const { quantizedMatrix, scale } = quantizeMatrix(fetch(name), dims[0], dims[1]);
+      native.modelSetTensor(handle, name + ".q", quantizedMatrix);
+      native.modelSetTensor(handle, name + ".scale", scale);
+    } else {
+      native.modelSetTensor(handle, name, fetch(name));
+    }
+    return { name, dims };
   }
 
   directoryNames(params) {

@@ -36,34 +36,29 @@ class SimpleTokenizer extends Tokenizer {
   decode(arr) { return Array.from(arr).map((x) => this.decoder[x]).join(""); }
 }
 
-const range = (x, y) => {
-  const res = [];
-  for (let i = x; i < y; i++) res.push(i);
-  return res;
-};
-const ord = (x) => x.charCodeAt(0);
-
-const bytes_to_unicode = () => {
-  const bs = range(ord("!"), ord("~") + 1).concat(range(ord("¡"), ord("¬") + 1), range(ord("®"), ord("ÿ") + 1));
-  const cs = bs.slice();
-  let n = 0;
+// GPT-2's byte <-> printable-character table: the 188 bytes that print on their own ('!'..'~',
+// '\u00a1'..'\u00ac', '\u00ae'..'\u00ff') stand for themselves, the other 68 are given the code points
+// 256, 257, ... in ascending byte order. `order` lists the characters in the order the vocabulary
+// numbers them (the printable ones first), `map` is byte -> character.
+function byteSymbols() {
+  const printable = (b) => (b >= 0x21 && b <= 0x7e) || (b >= 0xa1 && b <= 0xac) || (b >= 0xae && b <= 0xff);
+  const map = {};
+  const order = [];
   for (let b = 0; b < 256; b++) {
-    if (!bs.includes(b)) {
-      bs.push(b);
-      cs.push(256 + n);
-      n = n + 1;
+    if (printable(b)) {
+      map[b] = String.fromCharCode(b);
+      order.push(map[b]);
     }
   }
-  const result = {};
-  bs.forEach((b, i) => { result[b] = String.fromCharCode(cs[i]); });
-  return { map: result, order: cs.map((c) => String.fromCharCode(c)) };
-};
-
-const get_pairs = (word) => {
-  const pairs = [];
-  for (let i = 1; i < word.length; i++) pairs.push([word[i - 1], word[i]]);
-  return pairs;
-};
+  let shifted = 0;
+  for (let b = 0; b < 256; b++) {
+    if (!printable(b)) {
+      map[b] = String.fromCharCode(256 + shifted++);
+      order.push(map[b]);
+    }
+  }
+  return { map, order };
+}
 
 class GPT2Tokenizer extends Tokenizer {
   constructor() {
@@ -74,7 +69,7 @@ class GPT2Tokenizer extends Tokenizer {
   async load(bpeFile, tokensFile) {
     const lines = fs.readFileSync(bpeFile, "utf8").split("\n");
     const bpe_merges = lines.slice(1).filter((x) => x.trim().length > 0).map((x) => x.split(/\s+/).filter((e) => e.length > 0));
-    const { map, order } = bytes_to_unicode();
+    const { map, order } = byteSymbols();
     this.byte_encoder = map;
     this.byte_decoder = {};
     Object.keys(map).forEach((b) => { this.byte_decoder[map[b]] = parseInt(b); });
@@ -108,43 +103,35 @@ class GPT2Tokenizer extends Tokenizer {
     return Buffer.from(text.split("").map((x) => this.byte_decoder[x])).toString("utf8");
   }
 
+  // Byte-pair merging of one pre-token: repeatedly the adjacent pair of symbols with the lowest
+  // merge rank is joined, every occurrence of it in one left-to-right sweep (a joined symbol does not
+  // take part in another join of the same sweep), until no adjacent pair has a rank.
   bpe(token) {
-    if (this.cache.has(token)) return this.cache.get(token);
-    let word = token.split("");
-    let pairs = get_pairs(word);
-    if (pairs.length === 0) return token;
-    while (true) {
-      // the pair with the lowest merge rank; pairs without a rank never win
-      let best = null, bestRank = Infinity;
-      for (const p of pairs) {
-        const r = this.bpe_ranks.get(p[0] + " " + p[1]);
-        if (r !== undefined && r < bestRank) { best = p; bestRank = r; }
+    const hit = this.cache.get(token);
+    if (hit !== undefined) return hit;
+    let symbols = Array.from(token);
+    while (symbols.length > 1) {
+      let rank = Infinity, at = -1;
+      for (let i = 0; i + 1 < symbols.length; i++) {
+        const r = this.bpe_ranks.get(symbols[i] + " " + symbols[i + 1]);
+        if (r !== undefined && r < rank) { rank = r; at = i; }
       }
-      if (best === null) break;
-      const [first, second] = best;
-      let new_word = [];
-      let i = 0;
-      while (i < word.length) {
-        const j = word.indexOf(first, i);
-        if (j === -1) {
-          new_word = new_word.concat(word.slice(i));
-          break;
-        }
-        new_word = new_word.concat(word.slice(i, j));
-        i = j;
-        if (word[i] === first && i < word.length - 1 && word[i + 1] === second) {
-          new_word.push(first + second);
-          i = i + 2;
+      if (at < 0) break;
+      const left = symbols[at], right = symbols[at + 1];
+      const merged = new Array(symbols.length);
+      let n = 0;
+      for (let i = 0; i < symbols.length; i++) {
+        if (i + 1 < symbols.length && symbols[i] === left && symbols[i + 1] === right) {
+          merged[n++] = left + right;
+          i++;
         } else {
-          new_word.push(word[i]);
-          i = i + 1;
+          merged[n++] = symbols[i];
         }
       }
-      word = new_word;
-      if (word.length === 1) break;
-      pairs = get_pairs(word);
+      merged.length = n;
+      symbols = merged;
     }
-    const out = word.join(" ");
+    const out = symbols.join(" ");
     this.cache.set(token, out);
     return out;
   }

@@ -21,7 +21,7 @@ import time
 
 import numpy as np
 
-from . import _lib, blocks, sampling
+from . import _lib, blocks, quantize, sampling
 from .blocks import (AttentionBlock, DeEmbedBlock, EmbedBlock, FastMatMulBlock, GeluBlock, LayerNormBlock,
                      ResidualBlock, SoftmaxBlock)
 
@@ -69,7 +69,11 @@ def read_tensor(weightsFolder, name, params):
 
 
 class GPT:
-    def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0, tokenization=None):
+    def __init__(self, folder, type="bpe", tensors=None, params=None, tokenizer=None, flags=0, device_index=0, tokenization=None,
+                 quantize=None):
+        """`quantize="int8"` (or `"quantize": "int8"` in params_gpt.json) turns the four fp32 linear weights of
+        every layer into the weight-only int8 form of other/int8-gemm.js while they are loaded
+        (quantize.quantizeMatrix, per-output-column absmax); embeddings, biases and LayerNorm stay fp32."""
         self.folder = folder
         self.tokenizerType = type
         self.initialized = False
@@ -88,6 +92,9 @@ class GPT:
         self._flags = flags
         self._device_index = device_index
         self._tokenization = tokenization
+        if quantize not in (None, "int8"):
+            raise ValueError('quantize must be None or "int8"')
+        self._quantize = quantize
         self._handle = None
         self._history = []
         self.lastGpuMs = 0.0
@@ -154,7 +161,9 @@ class GPT:
         weightsFolder = folder
         params = self.loadParameters(weightsFolder)
         names = sorted(self._tensors) if self._tensors is not None else None
-        int8 = names is not None and any(n.endswith(".weight.q") for n in names)
+        packed = names is not None and any(n.endswith(".weight.q") for n in names)
+        quantise = (self._quantize or params.get("quantize")) == "int8" and not packed
+        int8 = packed or quantise
         p = _lib.Params(params["n_layer"], params["n_head"], params["n_embd"], params["n_ctx"], params["vocab_size"],
                         1 if int8 else 0, params.get("max_prefill", 0), self._flags)
         h = C.c_uint64(0)
@@ -162,9 +171,18 @@ class GPT:
         self._handle = h.value
         if names is None:
             names = [n for n in self._directory_names(params)]
-        for n in names:
-            a = np.ascontiguousarray(self._fetch(weightsFolder, n, params))
+        def send(n, a):
+            a = np.ascontiguousarray(a)
             _lib.call("wgpt_model_set_tensor", self._handle, n.encode(), a.ctypes.data_as(C.c_void_p), a.nbytes)
+
+        for n in names:
+            a = self._fetch(weightsFolder, n, params)
+            if quantise and n.startswith("transformer.h.") and n.split(".", 3)[3] in _LINEAR:
+                q, scale = quantize.quantizeMatrix(a)
+                send(n + ".q", q)
+                send(n + ".scale", scale)
+            else:
+                send(n, a)
         _lib.call("wgpt_model_finalize", self._handle)
         return {"handle": self._handle}, params
 
