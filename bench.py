@@ -45,6 +45,40 @@ def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
                       f"token as GPT.run does, C restatement of the WGSL kernels with OpenMP"}
 
 
+# HBM bytes of one decode step, from rocprofv3 --pmc counter runs (FETCH_SIZE x the copy-probe factor + WRITE_SIZE)
+# on single-token launches of the persistent kernel: bytes, the contexts of the profiled launches, the profile that
+# holds the figures and the first 16 hex digits of the SHA-256 of the kernel's source file when it was profiled.
+MEASURED_TRAFFIC = {
+    "gpt2-117m": (520.2e6, (171, 202), "profiles/decode_persistent_gpt2-117m.md", "KERNEL_SHA_117M"),
+    "gpt2-345m": (1564.7e6, (555, 586), "profiles/decode_persistent_other_configs.md", "KERNEL_SHA_OTHER"),
+    "gpt2-774m": (3187.3e6, (107, 138), "profiles/decode_persistent_other_configs.md", "KERNEL_SHA_OTHER"),
+    "gpt2-1.5b-int8": (2209.7e6, (171, 202), "profiles/decode_persistent_other_configs.md", "KERNEL_SHA_OTHER"),
+}
+KERNEL_SOURCE = os.path.join(ROOT, "webgpt_amd", "csrc", "decode_persistent.hip")
+
+
+def measured_traffic(config, persistent, ctx_lo, ctx_hi):
+    """(bytes or None, where the figure comes from). A counter figure is reported only for the kernel it was
+    measured on (same source file) and for a run whose contexts overlap the profiled ones; otherwise the line
+    says why there is none, so a stale figure cannot pass for a measurement of this run."""
+    import hashlib
+    if not persistent or config not in MEASURED_TRAFFIC:
+        return None, "no counter run for this configuration and decode path"
+    nbytes, (lo, hi), profile, sha = MEASURED_TRAFFIC[config]
+    try:
+        now = hashlib.sha256(open(KERNEL_SOURCE, "rb").read()).hexdigest()[:16]
+    except OSError:
+        now = "source not found"
+    where = {"profile": profile, "contexts": [lo, hi], "kernel_source_sha256_16": sha}
+    if now != sha:
+        where["stale"] = f"kernel source is now {now}: counters not re-collected since it changed"
+        return None, where
+    if ctx_hi < lo or ctx_lo > hi:
+        where["skipped"] = f"this run's contexts {ctx_lo}..{ctx_hi} do not overlap the profiled ones"
+        return None, where
+    return nbytes, where
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,10 +175,7 @@ def main():
             persistent = False
     kernel_name = ("decode_persistent_kernel (one launch runs all timed steps; one step = one token)" if persistent
                    else "per-block kernels (all launches of one token)")
-    # measured with rocprofv3 --pmc on single-token launches of the host loop that follows 40 timed steps, i.e. at
-    # contexts 171..202 (117M, int8), 555..586 (345M), 107..138 (774M); profiles/decode_persistent_*.md
-    measured = {"gpt2-117m": 520.2e6, "gpt2-345m": 1564.7e6, "gpt2-774m": 3187.3e6, "gpt2-1.5b-int8": 2209.7e6}
-    traffic = measured.get(args.config) if (persistent and args.prompt is None) else None
+    traffic, traffic_from = measured_traffic(args.config, persistent, pos, pos + args.steps - 1)
     out = {
         "metric": "ms/token + achieved HBM GB/s, GPT-2 117M fp32 batch-1 decode" if args.config == "gpt2-117m"
                   else f"ms/token + achieved HBM GB/s, {args.config} batch-1 decode",
@@ -173,7 +204,7 @@ def main():
         "host_loop_ms_per_token": {"mean": round(float(np.mean(per_tok)), 4), "p50": round(float(np.median(per_tok)), 4),
                                    "note": "wgpt_decode per token incl. logits read-back over PCIe"} if per_tok else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_from": traffic_from,
                      "kernel": kernel_name,
                      "bytes_per_step": int(bytes_total / args.steps),
                      "note": "achieved = algorithmic bytes (weights + KV rows read) of the timed steps / HIP-event time of "
