@@ -71,6 +71,15 @@ int wgpt_sync(void);
  * and K % 4 == 0 (vec4 view, 219-220). bias = 0 adds none. */
 int wgpt_matmul_bias(int M, int N, int K, wgpt_buf A, wgpt_buf W, wgpt_buf bias, wgpt_buf C);
 
+/* wgpt_matmul_bias for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arithmetic and result as
+ * wgpt_matmul_bias for M <= 4 (the batch-1 matrix-vector product), but the ceil(K/64) * M * N partial sums live
+ * in a fixed 4 MiB array inside the library's code object (one copy per GPU, held until the process ends)
+ * instead of a grow-only hipMalloc: the call allocates and frees nothing. Fails with WGPT_ERR_ARG when M > 4 or
+ * when the partial sums exceed 1048576 floats. All calls on a GPU share that array: calls that overlap in time
+ * (from several threads or streams) race; the library's single stream orders calls made one after the other. */
+int wgpt_matmul_bias_noalloc(int M, int N, int K, wgpt_buf A, wgpt_buf W, wgpt_buf bias, wgpt_buf C);
+
 /* other/int8-gemm.js:117-229 with a per-output-column scale (file header line 4):
  * W[k,n] = float(int8) / 127.0f * scale[n], Wq packed [K, N/4] words. bias = 0 adds none. */
 int wgpt_matmul_bias_i8(int M, int N, int K, wgpt_buf A, wgpt_buf Wq, wgpt_buf scale, wgpt_buf bias, wgpt_buf C);

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "wgpt_copy": ([_u64, _sz, _u64, _sz, _sz], True),
     "wgpt_sync": ([], True),
     "wgpt_matmul_bias": ([_int, _int, _int, _u64, _u64, _u64, _u64], True),
+    "wgpt_matmul_bias_noalloc": ([_int, _int, _int, _u64, _u64, _u64, _u64], True),
     "wgpt_matmul_bias_i8": ([_int, _int, _int, _u64, _u64, _u64, _u64, _u64], True),
     "wgpt_dequant_i8": ([_int, _int, _u64, _u64, _u64], True),
     "wgpt_residual": ([_int, _int, _u64, _u64, _u64], True),

@@ -17,7 +17,7 @@ struct Scratch {
 };
 static Scratch g_scratch[5];
 
-static int scratch(int slot, size_t bytes, void** out) {
+static int grow_scratch(int slot, size_t bytes, void** out) {
   Scratch& s = g_scratch[slot];
   if (s.bytes < bytes) {
     if (s.ptr) {
@@ -42,6 +42,27 @@ void release_scratch() {
   }
 }
 
+// ---- workspace of the allocation-free matrix-vector entry point (wgpt_matmul_bias_noalloc) ----
+// A fixed array in the code object instead of a hipMalloc: NOALLOC_SCRATCH_FLOATS floats (4 MiB) that every GPU
+// the library runs on holds until the process ends. In host code the name `scratch` is only a stand-in for the
+// symbol, never a device address: the address of this device's copy comes from hipGetSymbolAddress, once per
+// device at wgpt_init (setup_noalloc_scratch), and only that pointer is handed to kernels.
+constexpr size_t NOALLOC_SCRATCH_FLOATS = (size_t)1 << 20;
+static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static float* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+int setup_noalloc_scratch(int device) {
+  if (device < 0 || device >= NOALLOC_MAX_DEVICES) return fail(WGPT_ERR_ARG, "device %d: no workspace slot (at most %d devices)", device, NOALLOC_MAX_DEVICES);
+  if (g_scratch_ptr[device]) return WGPT_OK;
+  float* ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr)
+    return fail(WGPT_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", device, e == hipSuccess ? "null address" : hipGetErrorString(e));
+  g_scratch_ptr[device] = ptr;
+  return WGPT_OK;
+}
+
 static bool overlaps(const void* a, size_t an, const void* b, size_t bn) {
   const char* x = (const char*)a;
   const char* y = (const char*)b;
@@ -53,12 +74,12 @@ static int matmul_dev(int M, int N, int K, const float* A, const float* W, const
   hipError_t e;
   if (M <= GEMV_MAX_ROWS) {
     void* ws;
-    int rc = scratch(0, sizeof(float) * gemv_workspace_floats(M, N, K), &ws);
+    int rc = grow_scratch(0, sizeof(float) * gemv_workspace_floats(M, N, K), &ws);
     if (rc) return rc;
     e = launch_gemv_kn(M, N, K, A, K, W, N, bias, C, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   } else {
     void* ws;
-    int rc = scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
+    int rc = grow_scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
     if (rc) return rc;
     e = launch_gemm(M, N, K, A, K, W, N, bias, C, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   }
@@ -95,6 +116,36 @@ int wgpt_matmul_bias(int M, int N, int K, wgpt_buf A, wgpt_buf W, wgpt_buf bias,
   return matmul_dev(M, N, K, a, w, b, c);
 }
 
+int wgpt_matmul_bias_noalloc(int M, int N, int K, wgpt_buf A, wgpt_buf W, wgpt_buf bias, wgpt_buf C) {
+  WGPT_REQUIRE_INIT();
+  if (M < 1 || N < 1 || K < 1) return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_noalloc: M, N, K must be positive");
+  if (M > GEMV_MAX_ROWS)
+    return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_noalloc: M = %d exceeds the %d rows of the matrix-vector path; use wgpt_matmul_bias", M, GEMV_MAX_ROWS);
+  if (N % 8 != 0) return fail(WGPT_ERR_ARG, "Cols must be divisible by 16.");  // instructions.js:158
+  if (K % 4 != 0) return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_noalloc: K must be divisible by 4");
+  const size_t need = gemv_workspace_floats(M, N, K);
+  if (need > NOALLOC_SCRATCH_FLOATS)
+    return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_noalloc: ceil(K/%d) * M * N = %zu partial sums exceed the fixed workspace of %zu floats; "
+                "use wgpt_matmul_bias", GEMV_KCHUNK, need, NOALLOC_SCRATCH_FLOATS);
+  float* ws = rt().device >= 0 && rt().device < NOALLOC_MAX_DEVICES ? g_scratch_ptr[rt().device] : nullptr;
+  if (!ws) return fail(WGPT_ERR_STATE, "wgpt_matmul_bias_noalloc: the fixed workspace of device %d was not set up by wgpt_init", rt().device);
+  const float* a = F(A, (size_t)M * K, "wgpt_matmul_bias_noalloc(A)");
+  const float* w = F(W, (size_t)K * N, "wgpt_matmul_bias_noalloc(W)");
+  float* c = F(C, (size_t)M * N, "wgpt_matmul_bias_noalloc(C)");
+  if (!a || !w || !c) return WGPT_ERR_ARG;
+  const float* b = nullptr;
+  if (bias) {
+    b = F(bias, N, "wgpt_matmul_bias_noalloc(bias)");
+    if (!b) return WGPT_ERR_ARG;
+  }
+  if (overlaps(c, sizeof(float) * (size_t)M * N, a, sizeof(float) * (size_t)M * K))
+    return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_noalloc: C must not alias A");
+  // Nothing of the workspace has to start at zero: the first kernel writes every partial sum the second one reads.
+  hipError_t e = launch_gemv_kn(M, N, K, a, K, w, N, b, c, N, EPI_NONE, nullptr, ws, rt().stream);
+  if (e != hipSuccess) return fail(WGPT_ERR_HIP, "matmul launch: %s", hipGetErrorString(e));
+  return WGPT_OK;
+}
+
 int wgpt_matmul_bias_i8(int M, int N, int K, wgpt_buf A, wgpt_buf Wq, wgpt_buf scale, wgpt_buf bias, wgpt_buf C) {
   WGPT_REQUIRE_INIT();
   if (M < 1 || N < 1 || K < 1) return fail(WGPT_ERR_ARG, "wgpt_matmul_bias_i8: M, N, K must be positive");
@@ -115,19 +166,19 @@ int wgpt_matmul_bias_i8(int M, int N, int K, wgpt_buf A, wgpt_buf Wq, wgpt_buf s
   hipError_t e;
   if (M <= GEMV_MAX_ROWS) {
     void* ws;
-    int rc = scratch(0, sizeof(float) * gemv_workspace_floats(M, N, K), &ws);
+    int rc = grow_scratch(0, sizeof(float) * gemv_workspace_floats(M, N, K), &ws);
     if (rc) return rc;
     e = launch_gemv_kn_i8(M, N, K, a, K, wq, N / 4, sc, b, c, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   } else if (M >= 16) {
     // Dense contraction on the matrix cores, words dequantised on their way into LDS (same arithmetic).
     void* ws;
-    int rc = scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
+    int rc = grow_scratch(0, sizeof(float) * gemm_workspace_floats(M, N), &ws);
     if (rc) return rc;
     e = launch_gemm_i8(M, N, K, a, K, wq, N / 4, sc, b, c, N, EPI_NONE, nullptr, (float*)ws, rt().stream);
   } else {
     // A few rows more than the matrix-vector kernel takes: dequantise once (same arithmetic), then the fp32 tile kernel.
     void* wf;
-    int rc = scratch(1, sizeof(float) * (size_t)K * N, &wf);
+    int rc = grow_scratch(1, sizeof(float) * (size_t)K * N, &wf);
     if (rc) return rc;
     e = launch_dequant_i8(K, N, wq, N / 4, sc, (float*)wf, N, rt().stream);
     if (e == hipSuccess) e = launch_gemm(M, N, K, a, K, (const float*)wf, N, b, c, N, EPI_NONE, nullptr, nullptr, rt().stream);
@@ -204,7 +255,7 @@ int wgpt_sample_topk(int V, int top_k, double temperature, double u, wgpt_buf lo
   const int k = top_k < V ? top_k : V;
   // scratch: [u | probs[k]] doubles, then [tok | ids[k]] ints
   void* ws;
-  int rc = scratch(4, sizeof(double) * (size_t)(1 + k) + sizeof(int32_t) * (size_t)(1 + k), &ws);
+  int rc = grow_scratch(4, sizeof(double) * (size_t)(1 + k) + sizeof(int32_t) * (size_t)(1 + k), &ws);
   if (rc) return rc;
   double* du = (double*)ws;
   double* dprobs = du + 1;
@@ -244,7 +295,7 @@ int wgpt_embed(const int32_t* idx, int T, int d, int V, wgpt_buf wte, wgpt_buf w
   float* po = F(out, (size_t)T * d, "wgpt_embed(out)");
   if (!pe || !pp || !po) return WGPT_ERR_ARG;
   void* didx;
-  int rc = scratch(2, sizeof(int32_t) * (size_t)T, &didx);
+  int rc = grow_scratch(2, sizeof(int32_t) * (size_t)T, &didx);
   if (rc) return rc;
   WGPT_HIP(hipMemcpyAsync(didx, idx, sizeof(int32_t) * (size_t)T, hipMemcpyHostToDevice, rt().stream));
   // idx is caller memory that may change once this returns: finish the copy first.
@@ -289,7 +340,7 @@ int wgpt_attention(int T, int d, float scale, int H, int hs, wgpt_buf x, wgpt_bu
   if (!px || !wq || !wk || !wv || !wo || !pbq || !pbk || !pbv || !pbo || !po) return WGPT_ERR_ARG;
   if (px == po) return fail(WGPT_ERR_ARG, "wgpt_attention: out must not alias x");
   void* tmp;
-  int rc = scratch(3, sizeof(float) * 4 * td, &tmp);
+  int rc = grow_scratch(3, sizeof(float) * 4 * td, &tmp);
   if (rc) return rc;
   float* Q = (float*)tmp;
   float* Km = Q + td;

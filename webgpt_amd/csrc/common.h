@@ -30,6 +30,9 @@ void* resolve(wgpt_buf h, size_t need, const char* what);
 
 // Frees the grow-only scratch buffers of the block entry points.
 void release_scratch();
+// Looks up this device's address of the fixed workspace of wgpt_matmul_bias_noalloc; called by wgpt_init
+// with `device` current.
+int setup_noalloc_scratch(int device);
 
 #define WGPT_HIP(call)                                                                      \
   do {                                                                                      \

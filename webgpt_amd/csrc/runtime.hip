@@ -96,6 +96,10 @@ int wgpt_init(int device) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(WGPT_ERR_STATE, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
   r.compute_units = prop.multiProcessorCount;
+  {
+    const int rc = setup_noalloc_scratch(device);
+    if (rc) return rc;
+  }
   WGPT_HIP(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
   r.device = device;
   r.ready = true;

@@ -30,7 +30,7 @@ void* g_lib = nullptr;
   X(wgpt_model_reset_cache) X(wgpt_model_position) X(wgpt_model_tap) X(wgpt_model_last_gpu_ms)          \
   X(wgpt_model_decode_bytes) X(wgpt_model_set_decode_mode) X(wgpt_model_destroy) X(wgpt_synth_normal)   \
   X(wgpt_synth_tokens) X(wgpt_synth_int8_packed) X(wgpt_synth_uniform) X(wgpt_synth_tensor_id)   \
-  X(wgpt_decode_sample) X(wgpt_sample_topk)
+  X(wgpt_decode_sample) X(wgpt_sample_topk) X(wgpt_matmul_bias_noalloc)
 
 #define DECL(name) decltype(&::name) p_##name = nullptr;
 WGPT_FUNCS(DECL)
@@ -173,6 +173,7 @@ FN(Copy) {  // (dst, dstOff, src, srcOff, bytes)
 }
 
 FN(MatmulBias) { Args a(env, info); int M = a.i32(0), N = a.i32(1), K = a.i32(2); uint64_t A = a.u64(3), W = a.u64(4), b = a.u64(5), C = a.u64(6); if (!a.ok) return nullptr; if (failed(env, p_wgpt_matmul_bias(M, N, K, A, W, b, C))) return nullptr; return undefined(env); }
+FN(MatmulBiasNoAlloc) { Args a(env, info); int M = a.i32(0), N = a.i32(1), K = a.i32(2); uint64_t A = a.u64(3), W = a.u64(4), b = a.u64(5), C = a.u64(6); if (!a.ok) return nullptr; if (failed(env, p_wgpt_matmul_bias_noalloc(M, N, K, A, W, b, C))) return nullptr; return undefined(env); }
 FN(MatmulBiasI8) { Args a(env, info); int M = a.i32(0), N = a.i32(1), K = a.i32(2); uint64_t A = a.u64(3), W = a.u64(4), s = a.u64(5), b = a.u64(6), C = a.u64(7); if (!a.ok) return nullptr; if (failed(env, p_wgpt_matmul_bias_i8(M, N, K, A, W, s, b, C))) return nullptr; return undefined(env); }
 FN(DequantI8) { Args a(env, info); int K = a.i32(0), N = a.i32(1); uint64_t q = a.u64(2), s = a.u64(3), w = a.u64(4); if (!a.ok) return nullptr; if (failed(env, p_wgpt_dequant_i8(K, N, q, s, w))) return nullptr; return undefined(env); }
 FN(Residual) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), y = a.u64(3), o = a.u64(4); if (!a.ok) return nullptr; if (failed(env, p_wgpt_residual(M, N, x, y, o))) return nullptr; return undefined(env); }
@@ -389,7 +390,7 @@ napi_value InitModule(napi_env env, napi_value exports) {
   const struct { const char* name; napi_callback fn; } table[] = {
       {"load", Load}, {"exports", Exports}, {"init", Init}, {"shutdown", Shutdown}, {"sync", Sync}, {"deviceInfo", DeviceInfo},
       {"alloc", Alloc}, {"free", Free}, {"upload", Upload}, {"download", Download}, {"copy", Copy},
-      {"wgpt_matmul_bias", MatmulBias}, {"wgpt_matmul_bias_i8", MatmulBiasI8}, {"wgpt_dequant_i8", DequantI8},
+      {"wgpt_matmul_bias", MatmulBias}, {"wgpt_matmul_bias_noalloc", MatmulBiasNoAlloc}, {"wgpt_matmul_bias_i8", MatmulBiasI8}, {"wgpt_dequant_i8", DequantI8},
       {"wgpt_residual", Residual}, {"wgpt_layernorm", LayerNorm}, {"wgpt_softmax", Softmax}, {"wgpt_gelu", Gelu},
       {"wgpt_embed", Embed}, {"wgpt_deembed", DeEmbed}, {"wgpt_attention", Attention},
       {"modelCreate", ModelCreate}, {"modelSetTensor", ModelSetTensor}, {"modelFinalize", ModelFinalize},
