@@ -32,6 +32,9 @@ def run(inst, shape):
 @pytest.mark.parametrize("M,N,K", [(1, 8, 4), (1, 768, 768), (1, 2304, 768), (1, 768, 3072), (1, 72, 100), (2, 64, 64),
                                    (3, 1600, 1600), (4, 384, 1536), (5, 8, 12), (7, 200, 36), (16, 768, 768),
                                    (128, 2304, 768), (65, 136, 260), (200, 768, 3072), (2048, 4096, 64), (2050, 4104, 40),
+                                   # short prompts: K split over the waves of a workgroup (32x32 and 16x16 blocks, ragged M,
+                                   # K steps that do not divide by the eight waves)
+                                   (17, 32, 128), (100, 1600, 1600), (250, 96, 3200), (33, 6400, 1600), (256, 384, 384), (31, 64, 144),
                                    # the two-group kernel: K split four ways, one tile per compute unit, ragged M and N
                                    # with an odd number of K steps, and the same shape with a ragged K (other kernel)
                                    (512, 1024, 1024), (512, 4096, 1024), (950, 2056, 96), (950, 2056, 100)])

@@ -97,22 +97,22 @@ def test_full_depth_decode_step_against_oracle(name):
     gpt = GPT(None, "bpe", tensors=tensors, params=params)
     gpt.initialize()
     w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
-    tokens = synth.tokens(22, "prompt", 17, cfg["vocab_size"])
-    want = {T: ref.forward(p, w, tokens[:T]) for T in (12, 13, 17)}
-    got = gpt.prefill(tokens[:12])
-    report = {"prefill": worst(got, want[12])}
-    assert close(got, want[12]), (name, "prefill", report)
+    tokens = synth.tokens(22, "prompt", 21, cfg["vocab_size"])
+    want = {T: ref.forward(p, w, tokens[:T]) for T in (16, 17, 21)}
+    got = gpt.prefill(tokens[:16])
+    report = {"prefill": worst(got, want[16])}
+    assert close(got, want[16]), (name, "prefill", report)
     out = {}
     for mode in (1, 0):
         gpt.set_decode_mode(mode)
-        gpt.prefill(tokens[:12])
-        out[mode] = [gpt.decode(int(tokens[12 + i])) for i in range(5)]       # positions 12..16
-        for i, T in ((0, 13), (4, 17)):
+        gpt.prefill(tokens[:16])
+        out[mode] = [gpt.decode(int(tokens[16 + i])) for i in range(5)]       # positions 16..20
+        for i, T in ((0, 17), (4, 21)):
             report[f"mode{mode}@{T}"] = worst(out[mode][i], want[T])
     print(f"\nfull-depth parity {name}: worst |err| / (1e-5 + 1e-4 |want|) = " +
           ", ".join(f"{k} {v:.3f}" for k, v in report.items()))
     for mode in (1, 0):
-        for i, T in ((0, 13), (4, 17)):
+        for i, T in ((0, 17), (4, 21)):
             assert close(out[mode][i], want[T]), (name, mode, T, report)
             assert greedy_ok(out[mode][i], want[T])
         # the persistent kernel against the per-block kernels directly (for int8: the factored column scale

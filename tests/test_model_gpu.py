@@ -48,6 +48,28 @@ def test_prefill_taps_and_logits(device, cfg, T):
     gpt.unloadBuffers()
 
 
+@pytest.mark.parametrize("name,n_layer,T", [("toy", 6, 16), ("toy", 6, 33), ("toy", 3, 200), ("gpt2-117m", 2, 128), ("gpt2-1.5b", 1, 50)])
+def test_short_prompt_prefill_against_oracle(device, name, n_layer, T):
+    # prompts of 16..256 tokens without taps take the five-launches-per-layer path (LayerNorm inside c_attn and c_fc,
+    # K split over the waves of a workgroup): logits and the cache rows it leaves, then a decode step on top of them
+    cfg = dict(synth.CONFIGS[name])
+    cfg["n_layer"] = n_layer
+    gpt, tensors = load(cfg, seed=23)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(9, "prompt", T + 1, cfg["vocab_size"])
+    want, _, want_kv = ref.forward(p, w, tokens[:T], want_taps=True, want_kv=True)
+    got = gpt.prefill(tokens[:T])
+    assert close(got, want), worst(got, want)
+    assert greedy_ok(got, want)
+    for i in range(n_layer):
+        assert close(gpt.tap(f"kv{i}_k"), want_kv[i, 0]), (i, worst(gpt.tap(f"kv{i}_k"), want_kv[i, 0]))
+        assert close(gpt.tap(f"kv{i}_v"), want_kv[i, 1])
+    got = gpt.decode(int(tokens[T]))
+    want = ref.forward(p, w, tokens)
+    assert close(got, want), worst(got, want)
+    gpt.unloadBuffers()
+
+
 def test_decode_equals_last_row_of_full_forward(device):
     # decode(t) with the KV cache must equal the reference's full-window recompute of tokens [0..t]
     cfg = dict(synth.CONFIGS["toy"])

@@ -81,6 +81,24 @@ constexpr int SAMPLE_MAX_V = 262144;
 constexpr int SAMPLE_MAX_K = 1024;
 hipError_t launch_sample_topk(int V, int k, double temperature, const double* u, const float* logits, int32_t* tok,
                               int32_t* out, int slot, int32_t* ids, double* probs, hipStream_t s);
+// ---- one decode token with one launch per block; every launch reads the cache position from *pos, so the same
+//      launches (recorded once as a HIP graph) serve every token ----
+// C[N] = epi(row(x)[K] . W + bias) in one launch and one pass over a decode slab (column c of W is S = ceil(K/256)
+// segments of 64 lanes x float4, or x one word of four int8, starting at item c * S). row_mode: GEMV_ROW_PLAIN uses x
+// as it is, GEMV_ROW_NORMALISE the LayerNorm of x without gamma and beta (a slab that holds diag(gamma) W, a bias
+// that holds bias + beta W), GEMV_ROW_LAYERNORM the LayerNorm with gamma and beta. With kv the key/value columns of
+// a q/k/v row also go to cache row *pos.
+enum { GEMV_ROW_PLAIN = 0, GEMV_ROW_NORMALISE = 1, GEMV_ROW_LAYERNORM = 2 };
+hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const float* scale, const float* x, int row_mode,
+                            const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,
+                            const KvAfter* kv, const int* pos, hipStream_t s);
+// x[d] = wte[tok[0]] + wpe[*pos]
+hipError_t launch_embed_at(const int32_t* tok, int d, const int* pos, const float* wte, const float* wpe, float* x, hipStream_t s);
+// Attention of the one query at position *pos (q[h*hs..]) over cache rows 0..*pos of a head-major cache [H][ctx][hs].
+hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc, float* out,
+                                   const int* pos, hipStream_t s);
+hipError_t launch_advance_position(int* pos, hipStream_t s);
+
 // tok[0] = argmax(logits[0..V)) with the lowest index on ties; also stored to out[slot].
 hipError_t launch_argmax(int V, const float* logits, int32_t* tok, int32_t* out, int slot, hipStream_t s);
 

@@ -53,6 +53,9 @@ __device__ __forceinline__ float gelu_ref(float x) {
   return r;
 }
 
+// The same for a slab word, whose four bytes are consecutive k of ONE column (scale in every component of sc).
+__device__ __forceinline__ float4 unpack_i8x4_k(int32_t word, const float4& sc);
+
 __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 
@@ -77,6 +80,7 @@ __device__ __forceinline__ float4 unpack_i8x4(int32_t word, const float4& sc) {
   r.w = __fdiv_rn((float)b3, 127.0f) * sc.w;
   return r;
 }
+__device__ __forceinline__ float4 unpack_i8x4_k(int32_t word, const float4& sc) { return unpack_i8x4(word, sc); }
 
 // ---------------------------------------------------------------------------
 // FastMatMulBlock for M <= 4 (batch-1 decode): C = A . W + bias,
@@ -866,8 +870,9 @@ __global__ __launch_bounds__(WG) void softmax_kernel(int N, const float* __restr
 // EmbedBlock, instructions.js:795-821: gather + positional add in one pass.
 __global__ __launch_bounds__(WG) void embed_kernel(const int32_t* __restrict__ idx, int d, int pos0,
                                                     const float* __restrict__ wte, const float* __restrict__ wpe,
-                                                    float* __restrict__ out) {
+                                                    float* __restrict__ out, const int* __restrict__ pos_dev = nullptr) {
   const int i = blockIdx.x;
+  if (pos_dev) pos0 = *pos_dev;
   const size_t tok = (size_t)idx[i];
   const float* e = wte + tok * d;
   const float* p = wpe + (size_t)(pos0 + i) * d;
@@ -913,14 +918,17 @@ __global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const floa
 // row) per workgroup, reading K and V rows 0..p of head h at Kc + h*hstride + j*ldkv. Masked
 // positions j > p get weight exactly 0 in the reference (exp(-1e9 - max) underflows),
 // so they are skipped rather than multiplied by zero.
+// With pos_dev the position of the first query comes from device memory (a replayed launch serves every position).
 __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk, float scale, const float* __restrict__ q,
                                                         int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
-                                                        size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
+                                                        size_t hstride, int ldkv, float* __restrict__ out, int ldo,
+                                                        const int* __restrict__ pos_dev = nullptr) {
   extern __shared__ __attribute__((aligned(16))) float scores[];
   __shared__ __attribute__((aligned(16))) float qs[256];  // read as float4
   __shared__ float red[1024];
   __shared__ float sh[NWAVE];
   const int h = blockIdx.x, i = blockIdx.y;
+  if (pos_dev) pos0 = *pos_dev;
   const int nkeys = pos0 + i + 1;
   const int tid = threadIdx.x;
   if (tid < hs) qs[tid] = q[(size_t)i * ldq + h * hs + tid];
@@ -930,17 +938,17 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   const float4 qv = act ? ld4(qs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
   const float* kbase = Kc + h * hstride + sub * 4;
   const float* vbase = Vc + h * hstride + sub * 4;
-  // four key rows per lane group requested before the first is used: one after the other, the ~24 rounds of a
+  // eight key rows per lane group requested before the first is used: one after the other, the ~24 rounds of a
   // 380-key context each waited a full memory round trip
-  for (int j0 = 0; j0 < nkeys; j0 += 4 * ngrp) {
-    float4 kv[4];
+  for (int j0 = 0; j0 < nkeys; j0 += 8 * ngrp) {
+    float4 kv[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) {
       const int j = j0 + u * ngrp + grp;
       kv[u] = (act && j < nkeys) ? ld4(kbase + (size_t)j * ldkv) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) {
       const int j = j0 + u * ngrp + grp;
       float part = (qv.x * kv[u].x + qv.y * kv[u].y) + (qv.z * kv[u].z + qv.w * kv[u].w);
       for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
@@ -963,12 +971,12 @@ __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   if (act) {
     int j = grp;
-    for (; j + 3 * ngrp < nkeys; j += 4 * ngrp) {
-      float4 vv[4];
+    for (; j + 7 * ngrp < nkeys; j += 8 * ngrp) {
+      float4 vv[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) vv[u] = ld4(vbase + (size_t)(j + u * ngrp) * ldkv);
+      for (int u = 0; u < 8; ++u) vv[u] = ld4(vbase + (size_t)(j + u * ngrp) * ldkv);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) fma4(acc, scores[j + u * ngrp], vv[u]);
+      for (int u = 0; u < 8; ++u) fma4(acc, scores[j + u * ngrp], vv[u]);
     }
     for (; j < nkeys; j += ngrp) fma4(acc, scores[j], ld4(vbase + (size_t)j * ldkv));
     st4(red + grp * hs + sub * 4, acc);
@@ -1251,6 +1259,140 @@ __global__ __launch_bounds__(NWV * 64) void attention_mfma_kernel(int Tq, int po
   }
 }
 
+// ---------------------------------------------------------------------------
+// One decode token with one launch per block of the layer (the path of every model shape, replayable as a HIP
+// graph: nothing in a launch depends on the position except through *pos).
+//
+// gemv_slab_kernel: FastMatMulBlock at M = 1 (instructions.js:248-314) in ONE launch and one pass. The weights
+// are read from the decode slabs, in which the K values of a column are contiguous (segments of 256: 64 lanes x
+// float4, or x one word of four int8; K zero-padded to S segments): a wave owns R whole columns, so a dot product
+// never leaves its wave, no partial sums pass through memory and the sum has one fixed order. Every workgroup
+// first builds the input row in LDS, with the LayerNormBlock in front of the product applied on the way
+// (instructions.js:451-550: layernorm_kernel's order of operations; each workgroup repeats the two reductions
+// over the few KB of the row rather than wait for a separate launch). fp32 slabs of c_attn and c_fc hold
+// diag(gamma) W and their bias holds bias + beta W, so for them the row is only normalised (ROW_NORMALISE);
+// int8 slabs take the full LayerNorm (ROW_LAYERNORM). int8 weights are dequantised one by one as the shader does,
+// float(q) / 127.0f * scale[n] (other/int8-gemm.js:126-132). Bias last, then GELU or the residual add; the key
+// and value columns of a q/k/v row also go to cache row *pos.
+// ---------------------------------------------------------------------------
+enum { ROW_PLAIN = 0, ROW_NORMALISE = 1, ROW_LAYERNORM = 2 };
+struct GemvSlabArgs {
+  int N, K, S;
+  const void* slab;
+  const float* scale;   // int8: per column
+  const float* x;       // [K]
+  int row_mode;
+  const float* gamma;
+  const float* beta;
+  const float* bias;
+  int epi;
+  const float* resid;   // [N], may alias C
+  float* C;             // [N]
+  float* Kc;            // null: no cache scatter
+  float* Vc;
+  int d, hs, ctx;
+  const int* pos;
+};
+
+typedef float nt_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4_stream(const float4* p) {  // read once per token: keep it out of the way of the row and the cache
+  const nt_f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4*>(p));
+  return make_float4(t.x, t.y, t.z, t.w);
+}
+
+template <int R, bool I8>
+__global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
+  constexpr int CH = 8;  // segments of a column requested at a time
+  extern __shared__ __attribute__((aligned(16))) float xs[];  // [S * 256]
+  __shared__ float sh[NWAVE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int k4 = a.K >> 2, s64 = a.S * 64;
+  float s1 = 0.f;
+  for (int i = tid; i < s64; i += WG) {
+    const float4 v = i < k4 ? ld4(a.x + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    st4(xs + 4 * i, v);
+    s1 += (v.x + v.y) + (v.z + v.w);
+  }
+  if (a.row_mode != ROW_PLAIN) {
+    const float mean = block_sum(s1, sh) / (float)a.K;
+    float q = 0.f;
+    for (int i = tid; i < k4; i += WG) {
+      const float4 v = ld4(xs + 4 * i);
+      const float e0 = v.x - mean, e1 = v.y - mean, e2 = v.z - mean, e3 = v.w - mean;
+      q += (e0 * e0 + e1 * e1) + (e2 * e2 + e3 * e3);
+    }
+    const float var = block_sum(q, sh) / (float)a.K;
+    const float stdev = sqrtf(var + 1e-5f);
+    for (int i = tid; i < k4; i += WG) {
+      const float4 v = ld4(xs + 4 * i);
+      float4 o = make_float4((v.x - mean) / stdev, (v.y - mean) / stdev, (v.z - mean) / stdev, (v.w - mean) / stdev);
+      if (a.row_mode == ROW_LAYERNORM) {
+        const float4 g = ld4(a.gamma + 4 * i), b = ld4(a.beta + 4 * i);
+        o = make_float4(g.x * o.x + b.x, g.y * o.y + b.y, g.z * o.z + b.z, g.w * o.w + b.w);
+      }
+      st4(xs + 4 * i, o);
+    }
+  }
+  __syncthreads();
+  const int col0 = (blockIdx.x * NWAVE + wave) * R;
+  if (col0 >= a.N) return;
+  float acc[R];
+  int col[R];
+  float4 sc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    acc[r] = 0.f;
+    col[r] = col0 + r < a.N ? col0 + r : a.N - 1;  // columns beyond N repeat the last one and are not stored
+    if (I8) {
+      const float s = a.scale[col[r]];
+      sc[r] = make_float4(s, s, s, s);
+    }
+  }
+  for (int c0 = 0; c0 < a.S; c0 += CH) {
+    // all requests of the chunk first (unconditional: a segment beyond S repeats the last one and meets zeros)
+    float4 wf[I8 ? 1 : R][I8 ? 1 : CH];
+    int wq[I8 ? R : 1][I8 ? CH : 1];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const int seg = c0 + j < a.S ? c0 + j : a.S - 1;
+        const size_t at = ((size_t)col[r] * a.S + seg) * 64 + lane;
+        if constexpr (I8) wq[r][j] = __builtin_nontemporal_load(static_cast<const int32_t*>(a.slab) + at);
+        else wf[r][j] = ld4_stream(static_cast<const float4*>(a.slab) + at);
+      }
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c0 + j < a.S) xv = ld4(xs + (c0 + j) * 256 + lane * 4);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float4 w;
+        if constexpr (I8) w = unpack_i8x4_k(wq[r][j], sc[r]);
+        else w = wf[r][j];
+        acc[r] += (w.x * xv.x + w.y * xv.y) + (w.z * xv.z + w.w * xv.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float v = wave_sum(acc[r]);
+    const int n = col0 + r;
+    if (lane == 0 && n < a.N) {
+      if (a.bias) v += a.bias[n];
+      if (a.epi == EPI_GELU) v = gelu_ref(v);
+      else if (a.epi == EPI_RESIDUAL) v += a.resid[n];
+      a.C[n] = v;
+      if (a.Kc && n >= a.d) {
+        const int which = n >= 2 * a.d, c = n - (1 + which) * a.d, h = c / a.hs, e = c - h * a.hs;
+        (which ? a.Vc : a.Kc)[((size_t)h * a.ctx + *a.pos) * a.hs + e] = v;
+      }
+    }
+  }
+}
+
+__global__ void advance_position_kernel(int* pos) { *pos += 1; }
+
 __global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* __restrict__ src, int lds,
                                                         float* __restrict__ dst, int ldd) {
   const int r = blockIdx.y;
@@ -1405,11 +1547,18 @@ __global__ __launch_bounds__(1024) void argmax_kernel(int V, const float* __rest
   __shared__ int bi[1024];
   float best = -INFINITY;
   int besti = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += 1024) {
-    const float v = logits[i];
-    if (v > best || besti == 0x7fffffff) {
-      best = v;
-      besti = i;
+  // eight loads in flight per thread (one after the other, V = 50257 took 16 us); ascending i, so ties keep the lowest index
+  for (int i0 = threadIdx.x; i0 < V; i0 += 8 * 1024) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = i0 + u * 1024 < V ? logits[i0 + u * 1024] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * 1024;
+      if (i < V && (v[u] > best || besti == 0x7fffffff)) {
+        best = v[u];
+        besti = i;
+      }
     }
   }
   bv[threadIdx.x] = best;
@@ -1677,6 +1826,46 @@ hipError_t launch_sample_topk(int V, int k, double temperature, const double* u,
   if (V < 1 || V > SAMPLE_MAX_V || k < 1 || k > SAMPLE_MAX_K) return hipErrorInvalidValue;
   if (V <= 65536) sample_topk_kernel<true><<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
   else sample_topk_kernel<false><<<1, 1024, 0, s>>>(V, k, temperature, u, logits, tok, out, slot, ids, probs);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const float* scale, const float* x, int row_mode,
+                            const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,
+                            const KvAfter* kv, const int* pos, hipStream_t s) {
+  if ((K & 3) || N < 1) return hipErrorInvalidValue;
+  const int S = cdiv(K, 256);
+  const size_t lds = sizeof(float) * (size_t)S * 256;
+  if (lds > 48 * 1024) return hipErrorInvalidValue;
+  GemvSlabArgs a{N, K, S, slab, scale, x, row_mode, gamma, beta, bias, epi, resid, C, kv ? kv->Kc : nullptr, kv ? kv->Vc : nullptr,
+                 kv ? kv->d : 0, kv ? kv->hs : 1, kv ? kv->ctx : 0, pos};
+  if (int8) {
+    if (N >= 4096) gemv_slab_kernel<4, true><<<cdiv(N, NWAVE * 4), WG, lds, s>>>(a);
+    else gemv_slab_kernel<2, true><<<cdiv(N, NWAVE * 2), WG, lds, s>>>(a);
+  } else {
+    if (N >= 2048) gemv_slab_kernel<2, false><<<cdiv(N, NWAVE * 2), WG, lds, s>>>(a);
+    else gemv_slab_kernel<1, false><<<cdiv(N, NWAVE), WG, lds, s>>>(a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_embed_at(const int32_t* tok, int d, const int* pos, const float* wte, const float* wpe, float* x, hipStream_t s) {
+  embed_kernel<<<1, WG, 0, s>>>(tok, d, 0, wte, wpe, x, pos);
+  return hipGetLastError();
+}
+
+hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc, float* out,
+                                   const int* pos, hipStream_t s) {
+  int lpk = 1;
+  while (lpk * 4 < hs) lpk <<= 1;
+  if (lpk > 64 || hs > 256 || (hs & 3)) return hipErrorInvalidValue;
+  const size_t smem = sizeof(float) * (size_t)ctx;  // scores of the longest context: the launch is the same at every position
+  if (smem > 48 * 1024) return hipErrorInvalidValue;
+  attention_kernel<<<dim3(H, 1), WG, smem, s>>>(0, hs, lpk, scale, q, 0, Kc, Vc, (size_t)ctx * hs, hs, out, 0, pos);
+  return hipGetLastError();
+}
+
+hipError_t launch_advance_position(int* pos, hipStream_t s) {
+  advance_position_kernel<<<1, 1, 0, s>>>(pos);
   return hipGetLastError();
 }
 

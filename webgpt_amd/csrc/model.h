@@ -49,14 +49,23 @@ struct Model {
   double* u_dev = nullptr;         // [ctx] uniform draws of the sampling loop
 
   // persistent whole-token decode (decode_mode 1): slab-layout weights, exchange buffers
+  bool slabs_ok = false;   // pa.slabs / pa.lparams are built (every shape)
   bool persist_ok = false;
   PersistentArgs pa{};
   int* perr = nullptr;       // device error word of the persistent kernel
   // pinned host words (hipHostMalloc): [0] the token of a single-step call on its way to the device,
-  // [1] the error word on its way back, so that a decode call needs one stream synchronisation
+  // [1] the error word on its way back, so that a decode call needs one stream synchronisation, [2] the cache position
+  // on its way to pos_dev
   int32_t* pin = nullptr;
   float* logits_pin = nullptr;  // pinned host copy of the logits of the last call (V floats)
   unsigned epoch = 0;        // last epoch published by earlier launches
+
+  // decode with one launch per block (decode_mode 0): the token's launches read the cache position from pos_dev and
+  // are recorded once as a HIP graph that every later token replays
+  int* pos_dev = nullptr;
+  hipGraph_t token_graph = nullptr;
+  hipGraphExec_t token_graph_exec = nullptr;
+  bool token_graph_tried = false;
 
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   float last_ms = 0.f;

@@ -197,16 +197,94 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
   return WGPT_OK;
 }
 
-// Prepares the persistent whole-token decode path: slab-layout copies of the linear
-// weights, the per-layer pointer table and the exchange buffers. Leaves
-// m->persist_ok false (and the per-block path in charge) for shapes it does not cover.
+// The launches of one decode token at cache position *m->pos_dev (decode mode 0: any model shape): embedding, then
+// per layer c_attn (LayerNorm of its input row on the way in, cache append on the way out), attention, c_proj
+// (+ residual), c_fc (LayerNorm in, GELU out), mlp c_proj (+ residual); the final LayerNorm, the vocabulary
+// projection of that row (instructions.js:849-856) and the position advanced by one. 5L + 4 launches, none of
+// which carries the position as an argument. The products read the decode slabs (a column's K values contiguous).
+static int token_launches(Model* m) {
+  hipStream_t s = rt().stream;
+  const int d = m->d, H = m->H, hs = m->hs, hid = 4 * d;
+  const float scale = (float)(1.0 / std::sqrt((double)hs));  // model.js:321
+  const bool i8 = m->p.weight_dtype == 1;
+  const PersistentArgs& a = m->pa;
+  const LayerParamOffsets po = layer_param_offsets(d);
+  const size_t lane_bytes = i8 ? sizeof(int32_t) : sizeof(float4);
+  // fp32 slabs carry the LayerNorm gains and their biases the LayerNorm biases: the row is only normalised
+  const int ln_mode = i8 ? GEMV_ROW_LAYERNORM : GEMV_ROW_NORMALISE;
+  LAUNCH(launch_embed_at(m->tok_dev, d, m->pos_dev, m->wte, m->wpe, m->x, s));
+  for (int li = 0; li < m->L; ++li) {
+    const LayerW& l = m->layers[li];
+    float* Kc = m->kv + ((size_t)li * 2 + 0) * m->ctx * d;
+    float* Vc = m->kv + ((size_t)li * 2 + 1) * m->ctx * d;
+    const KvAfter kva = {Kc, Vc, d, hs, m->ctx, 0};
+    const char* slab = static_cast<const char*>(a.slabs) + (size_t)li * a.slab_stride * lane_bytes;
+    const float* lp = a.lparams + (size_t)li * po.stride;
+    LAUNCH(launch_gemv_slab(3 * d, d, slab, i8, lp + po.sA, m->x, ln_mode, l.ln1_g, l.ln1_b, lp + po.bA, m->qkv, EPI_NONE, nullptr, &kva,
+                            m->pos_dev, s));
+    LAUNCH(launch_attention_decode(H, hs, m->ctx, scale, m->qkv, Kc, Vc, m->att, m->pos_dev, s));
+    LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, m->att, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
+                            EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s));
+    LAUNCH(launch_gemv_slab(hid, d, slab + a.slab_offD * lane_bytes, i8, lp + po.sD, m->x, ln_mode, l.ln2_g, l.ln2_b, lp + po.bD, m->h, EPI_GELU,
+                            nullptr, nullptr, m->pos_dev, s));
+    LAUNCH(launch_gemv_slab(d, hid, slab + a.slab_offE * lane_bytes, i8, lp + po.sE, m->h, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bE, m->x,
+                            EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s));
+  }
+  LAUNCH(launch_layernorm(1, d, m->x, d, m->lnf_g, m->lnf_b, m->ln, d, s));
+  LAUNCH(launch_vocab_gemv(m->V, d, m->ln, m->wte, m->logits, s));
+  LAUNCH(launch_advance_position(m->pos_dev, s));
+  return WGPT_OK;
+}
+
+// Sends the host's cache position to pos_dev (the start of a decode call of mode 0; the token launches advance it).
+static int upload_position(Model* m) {
+  m->pin[2] = m->pos;  // every earlier use of the word has completed: each call ends with a synchronisation
+  WGPT_HIP(hipMemcpyAsync(m->pos_dev, &m->pin[2], sizeof(int), hipMemcpyHostToDevice, rt().stream));
+  return WGPT_OK;
+}
+
+// One decode token of mode 0 at the position in pos_dev. The launches are recorded as a HIP graph at first use
+// (kernel nodes only) and replayed afterwards; WEBGPT_AMD_NO_GRAPH=1, or a failed capture, launches them one by one.
+static int decode_token_blocks(Model* m) {
+  hipStream_t s = rt().stream;
+  if (!m->slabs_ok) return fail(WGPT_ERR_STATE, "decode: the decode layouts of the model were not built");
+  if (!m->token_graph_tried) {
+    m->token_graph_tried = true;
+    const char* off = getenv("WEBGPT_AMD_NO_GRAPH");
+    if (!(off && off[0] == '1')) {
+      WGPT_HIP(hipStreamSynchronize(s));
+      // a recording run changes nothing on the device: what is recorded is replayed below
+      if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        const int rc = token_launches(m);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(s, &g);
+        if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
+          m->token_graph = g;
+        } else {
+          if (g) (void)hipGraphDestroy(g);
+          m->token_graph_exec = nullptr;
+          (void)hipGetLastError();
+        }
+      } else {
+        (void)hipGetLastError();
+      }
+    }
+  }
+  if (m->token_graph_exec) {
+    WGPT_HIP(hipGraphLaunch(m->token_graph_exec, s));
+    return WGPT_OK;
+  }
+  return token_launches(m);
+}
+
+// Prepares the decode paths: slab-layout copies of the linear weights and the per-layer parameter blocks
+// (any shape), then, for the shapes the persistent whole-token kernel is built for, its per-workgroup
+// parameter blocks and exchange buffers. Leaves m->persist_ok false (and the per-block path in charge) for
+// shapes the persistent kernel does not cover.
 static int setup_persistent(Model* m) {
   m->persist_ok = false;
   const int d = m->d, hid = 4 * d, G = PD_GRID, split = PD_SPLIT_LONG;  // (the exchange buffer of the larger split)
   const bool i8 = m->p.weight_dtype == 1;
-  if (m->hs != 64) return WGPT_OK;
-  if (rt().compute_units < G) return WGPT_OK;
-  if (!persistent_supports(d, m->H, m->ctx, m->p.weight_dtype)) return WGPT_OK;
   PersistentArgs& a = m->pa;
   a = PersistentArgs{};
   a.L = m->L; a.H = m->H; a.d = d; a.ctx = m->ctx; a.V = m->V;
@@ -258,6 +336,15 @@ static int setup_persistent(Model* m) {
       LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_b, l.fc_b, lp + po.bD, rt().stream));
     }
   }
+  a.slabs = slabs;
+  a.lparams = lparams;
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  m->slabs_ok = true;
+  // The slabs and the folded parameters serve both decode paths (the one-launch-per-block path reads a column of a
+  // slab as one contiguous run of K); what follows is for the persistent kernel and the shapes it is built for.
+  if (m->hs != 64) return WGPT_OK;
+  if (rt().compute_units < G) return WGPT_OK;
+  if (!persistent_supports(d, m->H, m->ctx, m->p.weight_dtype)) return WGPT_OK;
   float* colparams;
   if ((rc = dev_alloc(m, sizeof(float) * (size_t)m->L * PD_GRID * PD_COLP, (void**)&colparams))) return rc;
   LAUNCH(build_colparams(lparams, m->L, d, i8 ? 1 : 0, colparams, rt().stream));
@@ -395,6 +482,8 @@ static int finish_timed(Model* m, float* logits) {
 }
 
 static void destroy_model(Model* m) {
+  if (m->token_graph_exec) (void)hipGraphExecDestroy(m->token_graph_exec);
+  if (m->token_graph) (void)hipGraphDestroy(m->token_graph);
   for (void* p : m->allocs) (void)hipFree(p);
   if (m->pin) (void)hipHostFree(m->pin);
   if (m->logits_pin) (void)hipHostFree(m->logits_pin);
@@ -483,10 +572,12 @@ int wgpt_model_finalize(wgpt_model h) {
   if ((rc = dev_alloc(m, (size_t)m->V * f, (void**)&m->logits))) return rc;
   if ((rc = dev_alloc(m, T * sizeof(int32_t), (void**)&m->tok_dev))) return rc;
   if (!m->pin) {
-    WGPT_HIP(hipHostMalloc((void**)&m->pin, 2 * sizeof(int32_t), hipHostMallocDefault));
-    m->pin[0] = m->pin[1] = 0;
+    WGPT_HIP(hipHostMalloc((void**)&m->pin, 4 * sizeof(int32_t), hipHostMallocDefault));
+    m->pin[0] = m->pin[1] = m->pin[2] = m->pin[3] = 0;
     WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * (size_t)m->V, hipHostMallocDefault));
   }
+  if ((rc = dev_alloc(m, sizeof(int), (void**)&m->pos_dev))) return rc;
+  WGPT_HIP(hipMemsetAsync(m->pos_dev, 0, sizeof(int), rt().stream));
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_samp_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(double), (void**)&m->u_dev))) return rc;
@@ -541,8 +632,10 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   if (m->pos >= m->ctx) return fail(WGPT_ERR_STATE, "wgpt_decode: context of %d positions is full; prefill a slid window", m->ctx);
   m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
   WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
+  int rc;
+  if (m->decode_mode != 1 && (rc = upload_position(m))) return rc;
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  int rc = m->decode_mode == 1 ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+  rc = m->decode_mode == 1 ? decode_persistent(m, 1) : decode_token_blocks(m);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
@@ -562,14 +655,18 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
     return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
   m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
   WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
-  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   const bool persistent = m->decode_mode == 1;
+  if (!persistent) {
+    int rc = upload_position(m);
+    if (rc) return rc;
+  }
+  WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   if (persistent) {
     int rc = decode_persistent(m, steps);
     if (rc) return rc;
   } else {
     for (int i = 0; i < steps; ++i) {
-      int rc = forward_blocks(m, 1, m->pos + i, false);
+      int rc = decode_token_blocks(m);  // advances the device's position itself
       if (rc) return rc;
       LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
     }
@@ -605,9 +702,13 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
     return fail(WGPT_ERR_STATE, "wgpt_decode_sample: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
   WGPT_HIP(hipMemcpyAsync(m->tok_dev, &token, sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   WGPT_HIP(hipMemcpyAsync(m->u_dev, u, sizeof(double) * (size_t)steps, hipMemcpyHostToDevice, rt().stream));
+  const bool persistent = m->decode_mode == 1;
+  if (!persistent) {
+    int rc0 = upload_position(m);
+    if (rc0) return rc0;
+  }
   WGPT_HIP(hipStreamSynchronize(rt().stream));
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  const bool persistent = m->decode_mode == 1;
   const int k = top_k < m->V ? top_k : m->V;
   // up to PD_TOPK candidates the persistent kernel selects and samples itself, all steps in one launch
   const bool in_kernel = persistent && k <= PD_TOPK;
@@ -621,7 +722,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   } else {
     for (int i = 0; i < steps && rc == WGPT_OK; ++i) {
       // one token per launch: the sampled id in tok_dev[0] is the next launch's input
-      rc = persistent ? decode_persistent(m, 1) : forward_blocks(m, 1, m->pos, false);
+      rc = persistent ? decode_persistent(m, 1) : decode_token_blocks(m);
       if (rc == WGPT_OK) {
         hipError_t e = launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream);
         if (e != hipSuccess) rc = fail(WGPT_ERR_HIP, "launch_sample_topk: %s", hipGetErrorString(e));
