@@ -325,3 +325,38 @@ def test_expired_wait_in_decode_sample_leaves_the_position_unchanged(device, mon
     _lib.call("wgpt_model_position", gpt._handle, C.byref(pos))
     assert pos.value == 11
     gpt.unloadBuffers()
+
+
+@pytest.mark.parametrize("name,dtype", [("toy", "f32"), ("toy", "int8")])
+def test_per_block_decode_graph_replays_equal_eager_launches(device, monkeypatch, name, dtype):
+    """Decode mode 0 records the launches of a token as a HIP graph (kernel nodes only; the position is read from
+    device memory) and replays it for every later token. Every replay, with eager prefills, host loops and
+    synchronisations between them, must give what the same launches give when issued one by one
+    (WEBGPT_AMD_NO_GRAPH=1), bit for bit, and both must match the oracle."""
+    cfg = dict(synth.CONFIGS[name])
+    cfg["n_layer"], cfg["dtype"] = 3, dtype
+    tokens = synth.tokens(31, "prompt", 40, cfg["vocab_size"])
+    out = {}
+    for graph in (True, False):
+        if not graph:
+            monkeypatch.setenv("WEBGPT_AMD_NO_GRAPH", "1")
+        gpt, tensors = load(cfg, seed=29)
+        gpt.set_decode_mode(0)
+        res = []
+        gpt.prefill(tokens[:9])
+        res += [gpt.decode(int(tokens[9 + i])) for i in range(6)]            # six replays, a read-back after each
+        ids = gpt.decode_greedy(int(tokens[15]), 5)                          # five replays in one call
+        res.append(np.asarray(ids, np.float32))
+        gpt.prefill(tokens[:20])                                             # eager work in between
+        res += [gpt.decode(int(tokens[20 + i])) for i in range(4)]
+        res.append(np.asarray(gpt.decode_sample(int(tokens[24]), 4, 3, 0.9, np.array([0.1, 0.5, 0.7, 0.95])), np.float32))
+        out[graph] = res
+        if graph:
+            w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+            want = ref.forward(p, w, tokens[:24])
+            assert close(res[10], want), worst(res[10], want)
+        gpt.unloadBuffers()
+        monkeypatch.delenv("WEBGPT_AMD_NO_GRAPH", raising=False)
+    assert len(out[True]) == len(out[False])
+    for i, (a, b) in enumerate(zip(out[True], out[False])):
+        assert np.array_equal(a, b), i

@@ -97,7 +97,9 @@ hipError_t launch_embed_at(const int32_t* tok, int d, const int* pos, const floa
 // Attention of the one query at position *pos (q[h*hs..]) over cache rows 0..*pos of a head-major cache [H][ctx][hs].
 hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc, float* out,
                                    const int* pos, hipStream_t s);
-hipError_t launch_advance_position(int* pos, hipStream_t s);
+// logits[v] = LayerNorm(x) . wte[v,:], then *pos += 1: the end of a decode token.
+hipError_t launch_vocab_gemv_ln(int V, int d, const float* x, const float* gamma, const float* beta, const float* wte, float* logits,
+                                int* pos, hipStream_t s);
 
 // tok[0] = argmax(logits[0..V)) with the lowest index on ties; also stored to out[slot].
 hipError_t launch_argmax(int V, const float* logits, int32_t* tok, int32_t* out, int slot, hipStream_t s);

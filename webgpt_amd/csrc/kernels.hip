@@ -4,6 +4,8 @@
 // reduction and combine by wave shuffles), which stays inside the fp32 tolerance.
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace wgpt {
 
 namespace {
@@ -918,17 +920,14 @@ __global__ __launch_bounds__(WG) void vocab_gemv_kernel(int V, int d, const floa
 // row) per workgroup, reading K and V rows 0..p of head h at Kc + h*hstride + j*ldkv. Masked
 // positions j > p get weight exactly 0 in the reference (exp(-1e9 - max) underflows),
 // so they are skipped rather than multiplied by zero.
-// With pos_dev the position of the first query comes from device memory (a replayed launch serves every position).
 __global__ __launch_bounds__(WG) void attention_kernel(int pos0, int hs, int lpk, float scale, const float* __restrict__ q,
                                                         int ldq, const float* __restrict__ Kc, const float* __restrict__ Vc,
-                                                        size_t hstride, int ldkv, float* __restrict__ out, int ldo,
-                                                        const int* __restrict__ pos_dev = nullptr) {
+                                                        size_t hstride, int ldkv, float* __restrict__ out, int ldo) {
   extern __shared__ __attribute__((aligned(16))) float scores[];
   __shared__ __attribute__((aligned(16))) float qs[256];  // read as float4
   __shared__ float red[1024];
   __shared__ float sh[NWAVE];
   const int h = blockIdx.x, i = blockIdx.y;
-  if (pos_dev) pos0 = *pos_dev;
   const int nkeys = pos0 + i + 1;
   const int tid = threadIdx.x;
   if (tid < hs) qs[tid] = q[(size_t)i * ldq + h * hs + tid];
@@ -1302,11 +1301,40 @@ __device__ __forceinline__ float4 ld4_stream(const float4* p) {  // read once pe
 
 template <int R, bool I8>
 __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
-  constexpr int CH = 8;  // segments of a column requested at a time
+  constexpr int CH = 8;  // segments of a column requested at a time (two register sets of this many)
   extern __shared__ __attribute__((aligned(16))) float xs[];  // [S * 256]
   __shared__ float sh[NWAVE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int k4 = a.K >> 2, s64 = a.S * 64;
+  // This wave's columns (beyond N: the last one again, never stored) and the first chunk of their weights, which
+  // do not depend on the row: requested before the row is built, so that they travel during the LayerNorm.
+  const int col0 = (blockIdx.x * NWAVE + wave) * R;
+  typedef typename std::conditional<I8, int32_t, float4>::type Item;
+  const Item* base[R];
+  float4 sc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int col = col0 + r < a.N ? col0 + r : a.N - 1;
+    base[r] = static_cast<const Item*>(a.slab) + (size_t)col * a.S * 64 + lane;
+    if (I8) {
+      const float s = a.scale[col];
+      sc[r] = make_float4(s, s, s, s);
+    }
+  }
+  Item w0[R][CH], w1[R][CH];
+  auto request = [&](Item (&w)[R][CH], int c0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        // unconditional: a segment beyond S repeats the last one and meets zeros
+        const int seg = c0 + j < a.S ? c0 + j : a.S - 1;
+        if constexpr (I8) w[r][j] = __builtin_nontemporal_load(base[r] + (size_t)seg * 64);
+        else w[r][j] = ld4_stream(base[r] + (size_t)seg * 64);
+      }
+  };
+  request(w0, 0);
+
   float s1 = 0.f;
   for (int i = tid; i < s64; i += WG) {
     const float4 v = i < k4 ? ld4(a.x + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1334,44 +1362,29 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
     }
   }
   __syncthreads();
-  const int col0 = (blockIdx.x * NWAVE + wave) * R;
-  if (col0 >= a.N) return;
   float acc[R];
-  int col[R];
-  float4 sc[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    acc[r] = 0.f;
-    col[r] = col0 + r < a.N ? col0 + r : a.N - 1;  // columns beyond N repeat the last one and are not stored
-    if (I8) {
-      const float s = a.scale[col[r]];
-      sc[r] = make_float4(s, s, s, s);
-    }
-  }
-  for (int c0 = 0; c0 < a.S; c0 += CH) {
-    // all requests of the chunk first (unconditional: a segment beyond S repeats the last one and meets zeros)
-    float4 wf[I8 ? 1 : R][I8 ? 1 : CH];
-    int wq[I8 ? R : 1][I8 ? CH : 1];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int j = 0; j < CH; ++j) {
-        const int seg = c0 + j < a.S ? c0 + j : a.S - 1;
-        const size_t at = ((size_t)col[r] * a.S + seg) * 64 + lane;
-        if constexpr (I8) wq[r][j] = __builtin_nontemporal_load(static_cast<const int32_t*>(a.slab) + at);
-        else wf[r][j] = ld4_stream(static_cast<const float4*>(a.slab) + at);
-      }
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  auto contract = [&](const Item (&w)[R][CH], int c0) {
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
       if (c0 + j < a.S) xv = ld4(xs + (c0 + j) * 256 + lane * 4);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        float4 w;
-        if constexpr (I8) w = unpack_i8x4_k(wq[r][j], sc[r]);
-        else w = wf[r][j];
-        acc[r] += (w.x * xv.x + w.y * xv.y) + (w.z * xv.z + w.w * xv.w);
+        float4 wv;
+        if constexpr (I8) wv = unpack_i8x4_k(w[r][j], sc[r]);
+        else wv = w[r][j];
+        acc[r] += (wv.x * xv.x + wv.y * xv.y) + (wv.z * xv.z + wv.w * xv.w);
       }
+    }
+  };
+  for (int c0 = 0; c0 < a.S; c0 += 2 * CH) {
+    if (c0 + CH < a.S) request(w1, c0 + CH);
+    contract(w0, c0);
+    if (c0 + CH < a.S) {
+      if (c0 + 2 * CH < a.S) request(w0, c0 + 2 * CH);
+      contract(w1, c0 + CH);
     }
   }
 #pragma unroll
@@ -1391,7 +1404,159 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
   }
 }
 
-__global__ void advance_position_kernel(int* pos) { *pos += 1; }
+// Attention of ONE query (the token being decoded, at cache position *pos) per head: formatQ + fusedWeights +
+// softmax + attentionValues of instructions.js:1129-1212 as attention_kernel computes them, arranged for the
+// latency of a single dependent chain: a workgroup per head requests the first 16 key rows AND value rows of each
+// of its lane groups (256 positions at head size 64) before anything else, so a context of up to 256 positions
+// costs one memory round trip; longer contexts continue in batches of the same size.
+__global__ __launch_bounds__(WG) void attention_decode_kernel(int hs, int lpk, int ctx, float scale, const float* __restrict__ q,
+                                                               const float* __restrict__ Kc, const float* __restrict__ Vc,
+                                                               size_t hstride, float* __restrict__ out, const int* __restrict__ pos) {
+  constexpr int U = 16;
+  extern __shared__ __attribute__((aligned(16))) float scores[];
+  __shared__ float red[1024];
+  __shared__ float sh[NWAVE];
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const int sub = tid & (lpk - 1), grp = tid / lpk, ngrp = WG / lpk;
+  const bool act = sub * 4 < hs;
+  const float* kbase = Kc + h * hstride + (act ? sub * 4 : 0);
+  const float* vbase = Vc + h * hstride + (act ? sub * 4 : 0);
+  // The first batch is requested before the position is known (rows up to the end of the cache exist; those
+  // beyond the context hold finite leftovers and are not used): its round trip overlaps that of *pos.
+  float4 k0[U], v0[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    int j = u * ngrp + grp;
+    j = j < ctx ? j : ctx - 1;
+    k0[u] = ld4(kbase + (size_t)j * hs);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    int j = u * ngrp + grp;
+    j = j < ctx ? j : ctx - 1;
+    v0[u] = ld4(vbase + (size_t)j * hs);
+  }
+  const int nkeys = *pos + 1;
+  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int j = u * ngrp + grp;
+    float part = (qv.x * k0[u].x + qv.y * k0[u].y) + (qv.z * k0[u].z + qv.w * k0[u].w);
+    for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
+    if (sub == 0 && j < nkeys) scores[j] = part * scale;
+  }
+  for (int j0 = U * ngrp; j0 < nkeys; j0 += U * ngrp) {
+    float4 kv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int j = j0 + u * ngrp + grp;
+      j = j < nkeys ? j : nkeys - 1;
+      kv[u] = ld4(kbase + (size_t)j * hs);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int j = j0 + u * ngrp + grp;
+      float part = (qv.x * kv[u].x + qv.y * kv[u].y) + (qv.z * kv[u].z + qv.w * kv[u].w);
+      for (int off = lpk >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off);
+      if (sub == 0 && j < nkeys) scores[j] = part * scale;
+    }
+  }
+  __syncthreads();
+  float m = -3.402823e+38f;
+  for (int j = tid; j < nkeys; j += WG) m = fmaxf(m, scores[j]);
+  m = block_max(m, sh);
+  float s = 0.f;
+  for (int j = tid; j < nkeys; j += WG) {
+    const float e = expf(scores[j] - m);
+    scores[j] = e;
+    s += e;
+  }
+  s = block_sum(s, sh);
+  for (int j = tid; j < nkeys; j += WG) scores[j] = scores[j] / s;
+  __syncthreads();
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int j = u * ngrp + grp;
+    if (j < nkeys) fma4(acc, scores[j], v0[u]);
+  }
+  for (int j0 = U * ngrp; j0 < nkeys; j0 += U * ngrp) {
+    float4 vv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int j = j0 + u * ngrp + grp;
+      j = j < nkeys ? j : nkeys - 1;
+      vv[u] = ld4(vbase + (size_t)j * hs);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int j = j0 + u * ngrp + grp;
+      if (j < nkeys) fma4(acc, scores[j], vv[u]);
+    }
+  }
+  if (act) st4(red + grp * hs + sub * 4, acc);
+  __syncthreads();
+  if (tid < hs) {
+    float o = 0.f;
+    for (int g = 0; g < ngrp; ++g) o += red[g * hs + tid];
+    out[h * hs + tid] = o;
+  }
+}
+
+// The final LayerNormBlock (model.js:224) and DeEmbedBlock (instructions.js:916-943) of a decode token in one
+// launch: every workgroup normalises the row itself while staging it (layernorm_kernel's order of operations), then
+// vocab_gemv_kernel's rows; the first workgroup finally advances the cache position (nothing later in the token
+// reads it).
+__global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const float* __restrict__ x, const float* __restrict__ gamma,
+                                                            const float* __restrict__ beta, const float* __restrict__ wte,
+                                                            float* __restrict__ logits, int* pos) {
+  extern __shared__ __attribute__((aligned(16))) float xs[];
+  __shared__ float sh[NWAVE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int v0 = (blockIdx.x * NWAVE + wave) * VOCAB_ROWS_PER_WAVE;
+  const int n4 = d >> 2;
+  float s1 = 0.f;
+  for (int c = threadIdx.x; c < n4; c += WG) {
+    const float4 v = ld4(x + 4 * c);
+    st4(xs + 4 * c, v);
+    s1 += (v.x + v.y) + (v.z + v.w);
+  }
+  const float mean = block_sum(s1, sh) / (float)d;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < n4; c += WG) {
+    const float4 v = ld4(xs + 4 * c);
+    const float e0 = v.x - mean, e1 = v.y - mean, e2 = v.z - mean, e3 = v.w - mean;
+    q += (e0 * e0 + e1 * e1) + (e2 * e2 + e3 * e3);
+  }
+  const float var = block_sum(q, sh) / (float)d;
+  const float stdev = sqrtf(var + 1e-5f);
+  for (int c = threadIdx.x; c < n4; c += WG) {
+    const float4 v = ld4(xs + 4 * c), g = ld4(gamma + 4 * c), b = ld4(beta + 4 * c);
+    st4(xs + 4 * c, make_float4(g.x * ((v.x - mean) / stdev) + b.x, g.y * ((v.y - mean) / stdev) + b.y,
+                                g.z * ((v.z - mean) / stdev) + b.z, g.w * ((v.w - mean) / stdev) + b.w));
+  }
+  __syncthreads();
+  float acc[VOCAB_ROWS_PER_WAVE];
+#pragma unroll
+  for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) acc[r] = 0.f;
+  for (int c = lane; c < n4; c += 64) {
+    const float4 xv = ld4(xs + 4 * c);
+#pragma unroll
+    for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+      if (v0 + r < V) {
+        const float4 w = ld4(wte + (size_t)(v0 + r) * d + 4 * c);
+        acc[r] += (xv.x * w.x + xv.y * w.y) + (xv.z * w.z + xv.w * w.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+    const float sum = wave_sum(acc[r]);
+    if (lane == 0 && v0 + r < V) logits[v0 + r] = sum;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) *pos += 1;
+}
+
 
 __global__ __launch_bounds__(WG) void copy_rows_kernel(int cols4, const float* __restrict__ src, int lds,
                                                         float* __restrict__ dst, int ldd) {
@@ -1860,12 +2025,14 @@ hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const fl
   if (lpk > 64 || hs > 256 || (hs & 3)) return hipErrorInvalidValue;
   const size_t smem = sizeof(float) * (size_t)ctx;  // scores of the longest context: the launch is the same at every position
   if (smem > 48 * 1024) return hipErrorInvalidValue;
-  attention_kernel<<<dim3(H, 1), WG, smem, s>>>(0, hs, lpk, scale, q, 0, Kc, Vc, (size_t)ctx * hs, hs, out, 0, pos);
+  attention_decode_kernel<<<H, WG, smem, s>>>(hs, lpk, ctx, scale, q, Kc, Vc, (size_t)ctx * hs, out, pos);
   return hipGetLastError();
 }
 
-hipError_t launch_advance_position(int* pos, hipStream_t s) {
-  advance_position_kernel<<<1, 1, 0, s>>>(pos);
+hipError_t launch_vocab_gemv_ln(int V, int d, const float* x, const float* gamma, const float* beta, const float* wte, float* logits,
+                                int* pos, hipStream_t s) {
+  const int rows_per_wg = NWAVE * VOCAB_ROWS_PER_WAVE;
+  vocab_gemv_ln_kernel<<<cdiv(V, rows_per_wg), WG, sizeof(float) * d, s>>>(V, d, x, gamma, beta, wte, logits, pos);
   return hipGetLastError();
 }
 

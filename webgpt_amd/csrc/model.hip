@@ -199,8 +199,8 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 
 // The launches of one decode token at cache position *m->pos_dev (decode mode 0: any model shape): embedding, then
 // per layer c_attn (LayerNorm of its input row on the way in, cache append on the way out), attention, c_proj
-// (+ residual), c_fc (LayerNorm in, GELU out), mlp c_proj (+ residual); the final LayerNorm, the vocabulary
-// projection of that row (instructions.js:849-856) and the position advanced by one. 5L + 4 launches, none of
+// (+ residual), c_fc (LayerNorm in, GELU out), mlp c_proj (+ residual); the final LayerNorm with the
+// vocabulary projection of that row (instructions.js:849-856), which also advances the position. 5L + 2 launches, none of
 // which carries the position as an argument. The products read the decode slabs (a column's K values contiguous).
 static int token_launches(Model* m) {
   hipStream_t s = rt().stream;
@@ -230,9 +230,7 @@ static int token_launches(Model* m) {
     LAUNCH(launch_gemv_slab(d, hid, slab + a.slab_offE * lane_bytes, i8, lp + po.sE, m->h, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bE, m->x,
                             EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s));
   }
-  LAUNCH(launch_layernorm(1, d, m->x, d, m->lnf_g, m->lnf_b, m->ln, d, s));
-  LAUNCH(launch_vocab_gemv(m->V, d, m->ln, m->wte, m->logits, s));
-  LAUNCH(launch_advance_position(m->pos_dev, s));
+  LAUNCH(launch_vocab_gemv_ln(m->V, d, m->x, m->lnf_g, m->lnf_b, m->wte, m->logits, m->pos_dev, s));
   return WGPT_OK;
 }
 
