@@ -1263,6 +1263,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       }
       __syncthreads();
       ++ep;
+      // Visibility of this token's cache rows to the next token. The slice that owned the new position appended k and v
+      // of every layer with write-through device-scope stores issued by wave 0; wave 0 also publishes this workgroup's
+      // word of the arg-max exchange below. Waiting here until every memory operation of the wave has completed
+      // (vmcnt = 0; the stores are tens of microseconds old, so the wait is free) orders them before that publish, and
+      // every workgroup polls every word of this exchange before it starts the next token: whoever reads these rows in a
+      // later step (slice boundaries move with the position, so it may be another workgroup) does so after they reached
+      // the level at which all compute units agree. Within the token the new row is read only by its writer, from LDS.
+      if (wave == 0) wait_loads();
       if (SAMPLE) {
         // the workgroup's K best of its waves' candidates (one per lane of wave 0), published in order
         if (wave == 0) {
