@@ -329,17 +329,17 @@ def test_expired_wait_in_decode_sample_leaves_the_position_unchanged(device, mon
 
 @pytest.mark.parametrize("name,dtype", [("toy", "f32"), ("toy", "int8")])
 def test_per_block_decode_graph_replays_equal_eager_launches(device, monkeypatch, name, dtype):
-    """Decode mode 0 records the launches of a token as a HIP graph (kernel nodes only; the position is read from
-    device memory) and replays it for every later token. Every replay, with eager prefills, host loops and
-    synchronisations between them, must give what the same launches give when issued one by one
-    (WEBGPT_AMD_NO_GRAPH=1), bit for bit, and both must match the oracle."""
+    """With WEBGPT_AMD_TOKEN_GRAPH=1 decode mode 0 records the launches of a token as a HIP graph (kernel nodes only; the
+    position is read from device memory) and replays it for every later token. Every replay, with eager prefills,
+    host loops and synchronisations between them, must give what the same launches give when issued one by one (the
+    default), bit for bit, and both must match the oracle."""
     cfg = dict(synth.CONFIGS[name])
     cfg["n_layer"], cfg["dtype"] = 3, dtype
     tokens = synth.tokens(31, "prompt", 40, cfg["vocab_size"])
     out = {}
     for graph in (True, False):
-        if not graph:
-            monkeypatch.setenv("WEBGPT_AMD_NO_GRAPH", "1")
+        if graph:
+            monkeypatch.setenv("WEBGPT_AMD_TOKEN_GRAPH", "1")
         gpt, tensors = load(cfg, seed=29)
         gpt.set_decode_mode(0)
         res = []
@@ -356,7 +356,7 @@ def test_per_block_decode_graph_replays_equal_eager_launches(device, monkeypatch
             want = ref.forward(p, w, tokens[:24])
             assert close(res[10], want), worst(res[10], want)
         gpt.unloadBuffers()
-        monkeypatch.delenv("WEBGPT_AMD_NO_GRAPH", raising=False)
+        monkeypatch.delenv("WEBGPT_AMD_TOKEN_GRAPH", raising=False)
     assert len(out[True]) == len(out[False])
     for i, (a, b) in enumerate(zip(out[True], out[False])):
         assert np.array_equal(a, b), i

@@ -241,15 +241,18 @@ static int upload_position(Model* m) {
   return WGPT_OK;
 }
 
-// One decode token of mode 0 at the position in pos_dev. The launches are recorded as a HIP graph at first use
-// (kernel nodes only) and replayed afterwards; WEBGPT_AMD_NO_GRAPH=1, or a failed capture, launches them one by one.
+// One decode token of mode 0 at the position in pos_dev. Because no launch carries the position, the token's launches
+// can be recorded once as a HIP graph (kernel nodes only) and replayed: WEBGPT_AMD_TOKEN_GRAPH=1 does that. It is
+// not the default: on MI355X the replay is exactly as fast as issuing the launches (117M: 0.4338 against 0.4326
+// ms/token; a token is bound by its 5L + 2 dependent kernels of 4-7 us each, not by the host), and rocprofv3 crashed
+// in its own graph handling on the 242-node graph of a 48-layer model.
 static int decode_token_blocks(Model* m) {
   hipStream_t s = rt().stream;
   if (!m->slabs_ok) return fail(WGPT_ERR_STATE, "decode: the decode layouts of the model were not built");
   if (!m->token_graph_tried) {
     m->token_graph_tried = true;
-    const char* off = getenv("WEBGPT_AMD_NO_GRAPH");
-    if (!(off && off[0] == '1')) {
+    const char* on = getenv("WEBGPT_AMD_TOKEN_GRAPH");
+    if (on && on[0] == '1') {
       WGPT_HIP(hipStreamSynchronize(s));
       // a recording run changes nothing on the device: what is recorded is replayed below
       if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
