@@ -50,8 +50,8 @@ def test_prefill_taps_and_logits(device, cfg, T):
 
 @pytest.mark.parametrize("name,n_layer,T", [("toy", 6, 16), ("toy", 6, 33), ("toy", 3, 200), ("gpt2-117m", 2, 128), ("gpt2-1.5b", 1, 50)])
 def test_short_prompt_prefill_against_oracle(device, name, n_layer, T):
-    # prompts of 16..256 tokens without taps take the five-launches-per-layer path (LayerNorm inside c_attn and c_fc,
-    # K split over the waves of a workgroup): logits and the cache rows it leaves, then a decode step on top of them
+    # prompts of 16..256 tokens run without taps (split-K products whose reduction pass applies the LayerNorm and
+    # scatters the cache rows): logits and the cache rows they leave, then a decode step on top of them
     cfg = dict(synth.CONFIGS[name])
     cfg["n_layer"] = n_layer
     gpt, tensors = load(cfg, seed=23)
