@@ -360,3 +360,37 @@ def test_per_block_decode_graph_replays_equal_eager_launches(device, monkeypatch
     assert len(out[True]) == len(out[False])
     for i, (a, b) in enumerate(zip(out[True], out[False])):
         assert np.array_equal(a, b), i
+
+
+@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("n_head,n_embd,n_ctx,start", [(2, 128, 600, 250), (3, 96, 1100, 1020)])
+def test_per_block_decode_across_cache_slices(device, monkeypatch, graph, n_head, n_embd, n_ctx, start):
+    """Decode mode 0 serves a context inside the first slice of the cache (256 positions at head size 64, 512 at 32)
+    with one workgroup per head and longer ones with a workgroup per (head, slice) whose results the attention
+    projection merges. Steps on both sides of the boundary, issued one by one and replayed as graphs, against the
+    oracle's full forward over the history (model.js:104-241)."""
+    cfg = small_cfg(n_layer=2, n_head=n_head, n_embd=n_embd, n_ctx=n_ctx, vocab_size=97)
+    if graph:
+        monkeypatch.setenv("WEBGPT_AMD_TOKEN_GRAPH", "1")
+    gpt, tensors = load(cfg, seed=37)
+    gpt.set_decode_mode(0)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(41, "prompt", start + 12, cfg["vocab_size"])
+    gpt.prefill(tokens[:start])
+    for i in range(12):
+        got = gpt.decode(int(tokens[start + i]))
+        if i in (0, 3, 4, 5, 6, 11):  # hs 64: 255 is the last position of the first slice; hs 32: 1024 the first of the third
+            want = ref.forward(p, w, tokens[:start + i + 1])
+            assert close(got, want), (i, worst(got, want))
+    ids = gpt.decode_greedy(int(np.argmax(got)), 3)
+    hist = [int(t) for t in tokens[:start + 12]] + [int(np.argmax(got))]
+    for t in ids:
+        lg = ref.forward(p, w, np.array(hist, np.int32))
+        assert int(np.argmax(lg)) == int(t) or greedy_gap_ok(lg, int(t)), (int(np.argmax(lg)), int(t))
+        hist.append(int(t))
+    gpt.unloadBuffers()
+
+
+def greedy_gap_ok(logits, chosen):
+    best = int(np.argmax(logits))
+    return abs(float(logits[best] - logits[chosen])) <= 1e-5 + 1e-4 * abs(float(logits[best]))

@@ -88,15 +88,28 @@ hipError_t launch_sample_topk(int V, int k, double temperature, const double* u,
 // as it is, GEMV_ROW_NORMALISE the LayerNorm of x without gamma and beta (a slab that holds diag(gamma) W, a bias
 // that holds bias + beta W), GEMV_ROW_LAYERNORM the LayerNorm with gamma and beta. With kv the key/value columns of
 // a q/k/v row also go to cache row *pos.
+// With merge (row_mode GEMV_ROW_PLAIN) the row is not x but the attention output that launch_attention_decode_slices
+// left in slices, combined while the row is staged.
 enum { GEMV_ROW_PLAIN = 0, GEMV_ROW_NORMALISE = 1, GEMV_ROW_LAYERNORM = 2 };
+struct AttnSlices {
+  float* part;  // [H][nslice][hs + 4]: unnormalised output, then the slice's maximum and sum
+  int nslice, hs;
+};
 hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const float* scale, const float* x, int row_mode,
                             const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,
-                            const KvAfter* kv, const int* pos, hipStream_t s);
+                            const KvAfter* kv, const int* pos, hipStream_t s, const AttnSlices* merge = nullptr);
 // x[d] = wte[tok[0]] + wpe[*pos]
 hipError_t launch_embed_at(const int32_t* tok, int d, const int* pos, const float* wte, const float* wpe, float* x, hipStream_t s);
 // Attention of the one query at position *pos (q[h*hs..]) over cache rows 0..*pos of a head-major cache [H][ctx][hs].
 hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc, float* out,
                                    const int* pos, hipStream_t s);
+// The same for a cache of more than one slice (attention_decode_slices(hs, ctx) > 1; a slice is 16 x 256 / lanes-per-key
+// positions, 256 at head size 64): a workgroup per (head, slice), results left in out->part for the merge of
+// launch_gemv_slab.
+int attention_decode_slice_positions(int hs);
+int attention_decode_slices(int hs, int ctx);
+hipError_t launch_attention_decode_slices(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc,
+                                          const AttnSlices* out, const int* pos, hipStream_t s);
 // logits[v] = LayerNorm(x) . wte[v,:], then *pos += 1: the end of a decode token.
 hipError_t launch_vocab_gemv_ln(int V, int d, const float* x, const float* gamma, const float* beta, const float* wte, float* logits,
                                 int* pos, hipStream_t s);

@@ -1274,7 +1274,7 @@ __global__ __launch_bounds__(NWV * 64) void attention_mfma_kernel(int Tq, int po
 // float(q) / 127.0f * scale[n] (other/int8-gemm.js:126-132). Bias last, then GELU or the residual add; the key
 // and value columns of a q/k/v row also go to cache row *pos.
 // ---------------------------------------------------------------------------
-enum { ROW_PLAIN = 0, ROW_NORMALISE = 1, ROW_LAYERNORM = 2 };
+enum { ROW_PLAIN = 0, ROW_NORMALISE = 1, ROW_LAYERNORM = 2, ROW_MERGE = 3 };
 struct GemvSlabArgs {
   int N, K, S;
   const void* slab;
@@ -1291,6 +1291,8 @@ struct GemvSlabArgs {
   float* Vc;
   int d, hs, ctx;
   const int* pos;
+  int nslice;           // ROW_MERGE: x holds [K / mhs][nslice][mhs + 4] attention slices
+  int mhs;
 };
 
 typedef float nt_f32x4 __attribute__((ext_vector_type(4)));
@@ -1301,7 +1303,9 @@ __device__ __forceinline__ float4 ld4_stream(const float4* p) {  // read once pe
 
 template <int R, bool I8>
 __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
-  constexpr int CH = 8;  // segments of a column requested at a time (two register sets of this many)
+  // segments of a column requested at a time (two register sets of this many): sized so that the kernel stays within
+  // 128 registers and two workgroups fit a compute unit (grids of 300-400 workgroups then run in one round)
+  constexpr int CH = (!I8 && R > 1) ? 4 : 8;
   extern __shared__ __attribute__((aligned(16))) float xs[];  // [S * 256]
   __shared__ float sh[NWAVE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1336,12 +1340,55 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
   request(w0, 0);
 
   float s1 = 0.f;
-  for (int i = tid; i < s64; i += WG) {
-    const float4 v = i < k4 ? ld4(a.x + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
-    st4(xs + 4 * i, v);
-    s1 += (v.x + v.y) + (v.z + v.w);
+  if (a.row_mode == ROW_MERGE) {
+    // the row is the attention output, still in slices of the context: (o[hs] unnormalised, max, sum) per head and
+    // slice, combined here as attention_decode_slice_kernel's header describes
+    const int stride = a.mhs + 4;
+    for (int i = tid; i < s64; i += WG) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < k4) {
+        const int h = (4 * i) / a.mhs, e = 4 * i - h * a.mhs;
+        const float* ph = a.x + (size_t)h * a.nslice * stride;
+        // eight slices at a time, everything requested before anything is used: one round trip, not one per slice
+        float mx = -3.402823e+38f, den = 0.f;
+        for (int s0 = 0; s0 < a.nslice; s0 += 8) {
+          float mv[8], lv[8];
+          float4 ov[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int sl = s0 + j < a.nslice ? s0 + j : a.nslice - 1;
+            mv[j] = ph[sl * stride + a.mhs];
+            lv[j] = ph[sl * stride + a.mhs + 1];
+            ov[j] = ld4(ph + sl * stride + e);
+          }
+          float mnew = mx;
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (s0 + j < a.nslice) mnew = fmaxf(mnew, mv[j]);
+          const float keep = expf(mx - mnew);  // rescales what earlier groups of eight have left
+          den *= keep;
+          v = make_float4(v.x * keep, v.y * keep, v.z * keep, v.w * keep);
+          mx = mnew;
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (s0 + j < a.nslice) {
+              const float w = expf(mv[j] - mx);
+              den += w * lv[j];
+              fma4(v, w, ov[j]);
+            }
+        }
+        v = make_float4(v.x / den, v.y / den, v.z / den, v.w / den);
+      }
+      st4(xs + 4 * i, v);
+    }
+  } else {
+    for (int i = tid; i < s64; i += WG) {
+      const float4 v = i < k4 ? ld4(a.x + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
+      st4(xs + 4 * i, v);
+      s1 += (v.x + v.y) + (v.z + v.w);
+    }
   }
-  if (a.row_mode != ROW_PLAIN) {
+  if (a.row_mode == ROW_NORMALISE || a.row_mode == ROW_LAYERNORM) {
     const float mean = block_sum(s1, sh) / (float)a.K;
     float q = 0.f;
     for (int i = tid; i < k4; i += WG) {
@@ -1500,6 +1547,92 @@ __global__ __launch_bounds__(WG) void attention_decode_kernel(int hs, int lpk, i
     float o = 0.f;
     for (int g = 0; g < ngrp; ++g) o += red[g * hs + tid];
     out[h * hs + tid] = o;
+  }
+}
+
+// The same attention for caches longer than one batch (U x WG / lpk positions: 256 at head size 64): the cache is cut
+// into fixed slices of that many positions, a workgroup per (head, slice), so every slice is one memory round trip
+// whatever the context, and a long context is read by several compute units instead of one. A slice leaves
+// (sum_j e_j v_j, m, sum_j e_j) with e_j = exp(score_j - m), m its own maximum (flash-decoding); a slice beyond the
+// context leaves (0, -FLT_MAX, 0). The consumer (gemv_slab_kernel, ROW_MERGE) combines them:
+// out = sum_s w_s o_s / sum_s w_s l_s with w_s = exp(m_s - max_s m_s), which is softmax(scores) . V of
+// instructions.js:1129-1212 in another order of summation.
+__global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int lpk, int ctx, float scale, const float* __restrict__ q,
+                                                                     const float* __restrict__ Kc, const float* __restrict__ Vc,
+                                                                     size_t hstride, float* __restrict__ part, const int* __restrict__ pos) {
+  constexpr int U = 16;
+  extern __shared__ __attribute__((aligned(16))) float scores[];  // [U * WG / lpk]
+  __shared__ float red[1024];
+  __shared__ float sh[NWAVE];
+  const int h = blockIdx.x, sl = blockIdx.y, nsl = gridDim.y, tid = threadIdx.x;
+  const int sub = tid & (lpk - 1), grp = tid / lpk, ngrp = WG / lpk;
+  const int j_lo = sl * U * ngrp;
+  const bool act = sub * 4 < hs;
+  const float* kbase = Kc + h * hstride + (act ? sub * 4 : 0);
+  const float* vbase = Vc + h * hstride + (act ? sub * 4 : 0);
+  // The first slice always has positions: it requests its rows before the position is known (rows up to the end of
+  // the cache exist), as attention_decode_kernel does. The others look at the position first: most of them are
+  // beyond the context most of the time, and their rows would be 3/4 of the launch's traffic for nothing.
+  int n_here = 0;
+  if (sl > 0) n_here = min(*pos + 1 - j_lo, U * ngrp);
+  float* dst = part + ((size_t)h * nsl + sl) * (hs + 4);
+  if (sl > 0 && n_here <= 0) {
+    if (tid < hs) dst[tid] = 0.f;
+    if (tid == 0) {
+      dst[hs] = -3.402823e+38f;
+      dst[hs + 1] = 0.f;
+    }
+    return;
+  }
+  float4 k0[U], v0[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    int j = j_lo + u * ngrp + grp;
+    j = j < ctx ? j : ctx - 1;
+    k0[u] = ld4(kbase + (size_t)j * hs);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    int j = j_lo + u * ngrp + grp;
+    j = j < ctx ? j : ctx - 1;
+    v0[u] = ld4(vbase + (size_t)j * hs);
+  }
+  if (sl == 0) n_here = min(*pos + 1, U * ngrp);  // positions of this slice inside the context
+  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int jl = u * ngrp + grp;
+    float p = (qv.x * k0[u].x + qv.y * k0[u].y) + (qv.z * k0[u].z + qv.w * k0[u].w);
+    for (int off = lpk >> 1; off > 0; off >>= 1) p += __shfl_xor(p, off);
+    if (sub == 0 && jl < n_here) scores[jl] = p * scale;
+  }
+  __syncthreads();
+  float m = -3.402823e+38f;
+  for (int j = tid; j < n_here; j += WG) m = fmaxf(m, scores[j]);
+  m = block_max(m, sh);
+  float l = 0.f;
+  for (int j = tid; j < n_here; j += WG) {
+    const float e = expf(scores[j] - m);
+    scores[j] = e;
+    l += e;
+  }
+  l = block_sum(l, sh);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int jl = u * ngrp + grp;
+    if (jl < n_here) fma4(acc, scores[jl], v0[u]);
+  }
+  if (act) st4(red + grp * hs + sub * 4, acc);
+  __syncthreads();
+  if (tid < hs) {
+    float o = 0.f;
+    for (int g = 0; g < ngrp; ++g) o += red[g * hs + tid];
+    dst[tid] = o;
+  }
+  if (tid == 0) {
+    dst[hs] = m;
+    dst[hs + 1] = l;
   }
 }
 
@@ -1996,13 +2129,15 @@ hipError_t launch_sample_topk(int V, int k, double temperature, const double* u,
 
 hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const float* scale, const float* x, int row_mode,
                             const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,
-                            const KvAfter* kv, const int* pos, hipStream_t s) {
+                            const KvAfter* kv, const int* pos, hipStream_t s, const AttnSlices* merge) {
   if ((K & 3) || N < 1) return hipErrorInvalidValue;
+  if (merge && (row_mode != GEMV_ROW_PLAIN || merge->nslice < 1 || merge->hs < 4 || (merge->hs & 3) || K % merge->hs)) return hipErrorInvalidValue;
   const int S = cdiv(K, 256);
   const size_t lds = sizeof(float) * (size_t)S * 256;
   if (lds > 48 * 1024) return hipErrorInvalidValue;
-  GemvSlabArgs a{N, K, S, slab, scale, x, row_mode, gamma, beta, bias, epi, resid, C, kv ? kv->Kc : nullptr, kv ? kv->Vc : nullptr,
-                 kv ? kv->d : 0, kv ? kv->hs : 1, kv ? kv->ctx : 0, pos};
+  GemvSlabArgs a{N, K, S, slab, scale, merge ? merge->part : x, merge ? (int)ROW_MERGE : row_mode, gamma, beta, bias, epi, resid, C,
+                 kv ? kv->Kc : nullptr, kv ? kv->Vc : nullptr, kv ? kv->d : 0, kv ? kv->hs : 1, kv ? kv->ctx : 0, pos,
+                 merge ? merge->nslice : 0, merge ? merge->hs : 1};
   if (int8) {
     if (N >= 4096) gemv_slab_kernel<4, true><<<cdiv(N, NWAVE * 4), WG, lds, s>>>(a);
     else gemv_slab_kernel<2, true><<<cdiv(N, NWAVE * 2), WG, lds, s>>>(a);
@@ -2026,6 +2161,27 @@ hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const fl
   const size_t smem = sizeof(float) * (size_t)ctx;  // scores of the longest context: the launch is the same at every position
   if (smem > 48 * 1024) return hipErrorInvalidValue;
   attention_decode_kernel<<<H, WG, smem, s>>>(hs, lpk, ctx, scale, q, Kc, Vc, (size_t)ctx * hs, out, pos);
+  return hipGetLastError();
+}
+
+int attention_decode_slice_positions(int hs) {
+  int lpk = 1;
+  while (lpk * 4 < hs) lpk <<= 1;
+  return lpk > 64 ? 0 : 16 * (WG / lpk);
+}
+
+int attention_decode_slices(int hs, int ctx) {
+  const int p = attention_decode_slice_positions(hs);
+  return p ? cdiv(ctx, p) : 0;
+}
+
+hipError_t launch_attention_decode_slices(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc,
+                                          const AttnSlices* out, const int* pos, hipStream_t s) {
+  int lpk = 1;
+  while (lpk * 4 < hs) lpk <<= 1;
+  if (lpk > 64 || hs > 256 || (hs & 3) || !out || out->hs != hs || out->nslice != attention_decode_slices(hs, ctx)) return hipErrorInvalidValue;
+  const size_t smem = sizeof(float) * 16 * (WG / lpk);
+  attention_decode_slice_kernel<<<dim3(H, out->nslice), WG, smem, s>>>(hs, lpk, ctx, scale, q, Kc, Vc, (size_t)ctx * hs, out->part, pos);
   return hipGetLastError();
 }
 

@@ -202,7 +202,7 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 // (+ residual), c_fc (LayerNorm in, GELU out), mlp c_proj (+ residual); the final LayerNorm with the
 // vocabulary projection of that row (instructions.js:849-856), which also advances the position. 5L + 2 launches, none of
 // which carries the position as an argument. The products read the decode slabs (a column's K values contiguous).
-static int token_launches(Model* m) {
+static int token_launches(Model* m, int pos) {
   hipStream_t s = rt().stream;
   const int d = m->d, H = m->H, hs = m->hs, hid = 4 * d;
   const float scale = (float)(1.0 / std::sqrt((double)hs));  // model.js:321
@@ -212,6 +212,10 @@ static int token_launches(Model* m) {
   const size_t lane_bytes = i8 ? sizeof(int32_t) : sizeof(float4);
   // fp32 slabs carry the LayerNorm gains and their biases the LayerNorm biases: the row is only normalised
   const int ln_mode = i8 ? GEMV_ROW_LAYERNORM : GEMV_ROW_NORMALISE;
+  // `pos` is what the host knows of the token's cache position; the launches themselves read it from the device. It
+  // only chooses the attention: a context that fits the first slice of the cache is served by the
+  // one-workgroup-per-head kernel, which costs a launch of H instead of H x slices workgroups and no merge.
+  const bool sliced = m->att_nslice > 1 && pos + 1 > attention_decode_slice_positions(hs);
   LAUNCH(launch_embed_at(m->tok_dev, d, m->pos_dev, m->wte, m->wpe, m->x, s));
   for (int li = 0; li < m->L; ++li) {
     const LayerW& l = m->layers[li];
@@ -222,9 +226,16 @@ static int token_launches(Model* m) {
     const float* lp = a.lparams + (size_t)li * po.stride;
     LAUNCH(launch_gemv_slab(3 * d, d, slab, i8, lp + po.sA, m->x, ln_mode, l.ln1_g, l.ln1_b, lp + po.bA, m->qkv, EPI_NONE, nullptr, &kva,
                             m->pos_dev, s));
-    LAUNCH(launch_attention_decode(H, hs, m->ctx, scale, m->qkv, Kc, Vc, m->att, m->pos_dev, s));
-    LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, m->att, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
-                            EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s));
+    if (sliced) {  // a workgroup per (head, slice of the cache), merged as c_proj stages its row
+      const AttnSlices sl = {m->att_part, m->att_nslice, hs};
+      LAUNCH(launch_attention_decode_slices(H, hs, m->ctx, scale, m->qkv, Kc, Vc, &sl, m->pos_dev, s));
+      LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, nullptr, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
+                              EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s, &sl));
+    } else {
+      LAUNCH(launch_attention_decode(H, hs, m->ctx, scale, m->qkv, Kc, Vc, m->att, m->pos_dev, s));
+      LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, m->att, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
+                              EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s));
+    }
     LAUNCH(launch_gemv_slab(hid, d, slab + a.slab_offD * lane_bytes, i8, lp + po.sD, m->x, ln_mode, l.ln2_g, l.ln2_b, lp + po.bD, m->h, EPI_GELU,
                             nullptr, nullptr, m->pos_dev, s));
     LAUNCH(launch_gemv_slab(d, hid, slab + a.slab_offE * lane_bytes, i8, lp + po.sE, m->h, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bE, m->x,
@@ -246,7 +257,7 @@ static int upload_position(Model* m) {
 // not the default: on MI355X the replay is exactly as fast as issuing the launches (117M: 0.4338 against 0.4326
 // ms/token; a token is bound by its 5L + 2 dependent kernels of 4-7 us each, not by the host), and rocprofv3 crashed
 // in its own graph handling on the 242-node graph of a 48-layer model.
-static int decode_token_blocks(Model* m) {
+static int decode_token_blocks(Model* m, int pos) {
   hipStream_t s = rt().stream;
   if (!m->slabs_ok) return fail(WGPT_ERR_STATE, "decode: the decode layouts of the model were not built");
   if (!m->token_graph_tried) {
@@ -254,28 +265,41 @@ static int decode_token_blocks(Model* m) {
     const char* on = getenv("WEBGPT_AMD_TOKEN_GRAPH");
     if (on && on[0] == '1') {
       WGPT_HIP(hipStreamSynchronize(s));
-      // a recording run changes nothing on the device: what is recorded is replayed below
-      if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
-        const int rc = token_launches(m);
-        hipGraph_t g = nullptr;
-        const hipError_t e = hipStreamEndCapture(s, &g);
-        if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
-          m->token_graph = g;
-        } else {
-          if (g) (void)hipGraphDestroy(g);
-          m->token_graph_exec = nullptr;
-          (void)hipGetLastError();
+      // One graph per attention variant (the context inside the first slice of the cache, or beyond it), so that a
+      // replay runs exactly the launches the host would issue. A recording run changes nothing on the device.
+      const int variants = m->att_nslice > 1 ? 2 : 1;
+      bool ok = true;
+      for (int v = 0; v < variants && ok; ++v) {
+        ok = false;
+        if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+          const int rc = token_launches(m, v == 0 ? 0 : m->ctx - 1);
+          hipGraph_t g = nullptr;
+          const hipError_t e = hipStreamEndCapture(s, &g);
+          if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec[v], g, nullptr, nullptr, 0) == hipSuccess) {
+            m->token_graph[v] = g;
+            ok = true;
+          } else if (g) {
+            (void)hipGraphDestroy(g);
+          }
         }
-      } else {
+      }
+      if (!ok) {  // issue the launches instead
+        for (int v = 0; v < 2; ++v) {
+          if (m->token_graph_exec[v]) (void)hipGraphExecDestroy(m->token_graph_exec[v]);
+          if (m->token_graph[v]) (void)hipGraphDestroy(m->token_graph[v]);
+          m->token_graph_exec[v] = nullptr;
+          m->token_graph[v] = nullptr;
+        }
         (void)hipGetLastError();
       }
     }
   }
-  if (m->token_graph_exec) {
-    WGPT_HIP(hipGraphLaunch(m->token_graph_exec, s));
+  if (m->token_graph_exec[0]) {
+    const bool sliced = m->att_nslice > 1 && pos + 1 > attention_decode_slice_positions(m->hs);
+    WGPT_HIP(hipGraphLaunch(m->token_graph_exec[sliced ? 1 : 0], s));
     return WGPT_OK;
   }
-  return token_launches(m);
+  return token_launches(m, pos);
 }
 
 // Prepares the decode paths: slab-layout copies of the linear weights and the per-layer parameter blocks
@@ -483,8 +507,10 @@ static int finish_timed(Model* m, float* logits) {
 }
 
 static void destroy_model(Model* m) {
-  if (m->token_graph_exec) (void)hipGraphExecDestroy(m->token_graph_exec);
-  if (m->token_graph) (void)hipGraphDestroy(m->token_graph);
+  for (int v = 0; v < 2; ++v) {
+    if (m->token_graph_exec[v]) (void)hipGraphExecDestroy(m->token_graph_exec[v]);
+    if (m->token_graph[v]) (void)hipGraphDestroy(m->token_graph[v]);
+  }
   for (void* p : m->allocs) (void)hipFree(p);
   if (m->pin) (void)hipHostFree(m->pin);
   if (m->logits_pin) (void)hipHostFree(m->logits_pin);
@@ -578,6 +604,8 @@ int wgpt_model_finalize(wgpt_model h) {
     WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * (size_t)m->V, hipHostMallocDefault));
   }
   if ((rc = dev_alloc(m, sizeof(int), (void**)&m->pos_dev))) return rc;
+  m->att_nslice = attention_decode_slices(m->hs, m->ctx);
+  if (m->att_nslice > 1 && (rc = dev_alloc(m, (size_t)m->H * m->att_nslice * (m->hs + 4) * f, (void**)&m->att_part))) return rc;
   WGPT_HIP(hipMemsetAsync(m->pos_dev, 0, sizeof(int), rt().stream));
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_tok_dev))) return rc;
   if ((rc = dev_alloc(m, (size_t)m->ctx * sizeof(int32_t), (void**)&m->out_samp_dev))) return rc;
@@ -636,7 +664,7 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   int rc;
   if (m->decode_mode != 1 && (rc = upload_position(m))) return rc;
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  rc = m->decode_mode == 1 ? decode_persistent(m, 1) : decode_token_blocks(m);
+  rc = m->decode_mode == 1 ? decode_persistent(m, 1) : decode_token_blocks(m, m->pos);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
@@ -667,7 +695,7 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
     if (rc) return rc;
   } else {
     for (int i = 0; i < steps; ++i) {
-      int rc = decode_token_blocks(m);  // advances the device's position itself
+      int rc = decode_token_blocks(m, m->pos + i);  // advances the device's position itself
       if (rc) return rc;
       LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
     }
@@ -723,7 +751,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   } else {
     for (int i = 0; i < steps && rc == WGPT_OK; ++i) {
       // one token per launch: the sampled id in tok_dev[0] is the next launch's input
-      rc = persistent ? decode_persistent(m, 1) : decode_token_blocks(m);
+      rc = persistent ? decode_persistent(m, 1) : decode_token_blocks(m, m->pos);
       if (rc == WGPT_OK) {
         hipError_t e = launch_sample_topk(m->V, k, temperature, m->u_dev + i, m->logits, m->tok_dev, m->out_samp_dev, i, nullptr, nullptr, rt().stream);
         if (e != hipSuccess) rc = fail(WGPT_ERR_HIP, "launch_sample_topk: %s", hipGetErrorString(e));
