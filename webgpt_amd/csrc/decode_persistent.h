@@ -68,6 +68,7 @@ struct PersistentArgs {
   // [4] residual row into c_fc, [5] hidden row, [6] arg-max candidates
   int delay[7];
   unsigned spin_limit;  // poll rounds after which a wait gives up and raises *err
+  int short_keys;       // a launch whose last step attends to more positions runs the instantiation with PD_SPLIT_LONG slices (<= PD_SHORT_KEYS)
   // token selection: top_k == 1 is the arg-max; 2..PD_TOPK samples as GPT.generate does
   // (model.js:81-85) with u[step] for the step's Math.random() and the float64 temperature
   int top_k;

@@ -1051,9 +1051,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // exp(m_s - M) / sum are made once (thread h * SPLIT + s; `part` is idle between the attention and the
         // next LayerNorm) and read back as broadcasts: every element deriving them itself cost SPLIT exponentials
         // per element, 1.45 us of the phase at d = 1600.
+        // (The fp32 d = 1600 shape, which lives on spilled registers, keeps the per-element form: with the extra
+        // barrier and the shared weights it ran 8 % slower, 1.585 -> 1.713 ms/token.)
         constexpr int MERGE_ROUNDS = (D + NT - 1) / NT;
+        constexpr bool MERGE_ONCE = I8 || D < 1600;
         static_assert(H * SPLIT <= NT && H * SPLIT <= PART, "one thread and one float of `part` per (head, slice)");
-        if (tid < H * SPLIT) {
+        if (MERGE_ONCE && tid < H * SPLIT) {
           const int h = tid / SPLIT;
           const float* phd = attp + h * SPLIT * (HS + 2);
           float ms[SPLIT];
@@ -1072,7 +1075,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
           part[tid] = mine * fast_rcp(Lsum);
         }
-        __syncthreads();
+        if (MERGE_ONCE) __syncthreads();
         const Leading<LoadD, SPN, SPD> leadD{nextD};
         static_for<MERGE_ROUNDS>([&](auto KK) {
           constexpr int k = decltype(KK)::value;
@@ -1080,11 +1083,29 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           if (k * NT + NT <= D || e < D) {
             const int h = e / HS, c = e - h * HS;
             const float* phd = attp + h * SPLIT * (HS + 2);
-            const float* wn = part + h * SPLIT;
-            float val = 0.f;
+            if constexpr (MERGE_ONCE) {
+              const float* wn = part + h * SPLIT;
+              float val = 0.f;
 #pragma unroll
-            for (int s2 = 0; s2 < SPLIT; ++s2) val += phd[s2 * (HS + 2) + c] * wn[s2];
-            xs1[e] = val;
+              for (int s2 = 0; s2 < SPLIT; ++s2) val += phd[s2 * (HS + 2) + c] * wn[s2];
+              xs1[e] = val;
+            } else {
+              float ms[SPLIT];
+              float M = -INFINITY;
+#pragma unroll
+              for (int s2 = 0; s2 < SPLIT; ++s2) {
+                ms[s2] = phd[s2 * (HS + 2) + HS];
+                M = fmaxf(M, ms[s2]);
+              }
+              float Lsum = 0.f, val = 0.f;
+#pragma unroll
+              for (int s2 = 0; s2 < SPLIT; ++s2) {
+                const float wv = ms[s2] > -INFINITY ? fast_exp(ms[s2] - M) : 0.f;
+                Lsum += phd[s2 * (HS + 2) + HS + 1] * wv;
+                val += phd[s2 * (HS + 2) + c] * wv;
+              }
+              xs1[e] = val * fast_rcp(Lsum);
+            }
           }
           // (the few dot products of this phase cannot take c_fc's requests between them: the rounds of the merge do)
           if constexpr (SPREAD) {
@@ -1548,7 +1569,8 @@ template <int D, int H, bool I8>
 hipError_t launch_t(const PersistentArgs& a, hipStream_t s) {
   const int keys = a.pos0 + a.nsteps;  // positions the last step attends to
   if (keys > 32 * PD_KVBATCH * PD_SPLIT_LONG) return hipErrorInvalidValue;
-  if (keys <= PD_SHORT_KEYS) return launch_kv<Shape<D, H, I8, PD_SPLIT>, PD_KVBATCH>(a, s);
+  if (a.short_keys < 0 || a.short_keys > PD_SHORT_KEYS) return hipErrorInvalidValue;
+  if (keys <= a.short_keys) return launch_kv<Shape<D, H, I8, PD_SPLIT>, PD_KVBATCH>(a, s);
   return launch_kv<Shape<D, H, I8, PD_SPLIT_LONG>, PD_KVBATCH>(a, s);
 }
 

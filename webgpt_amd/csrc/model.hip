@@ -421,6 +421,13 @@ static int setup_persistent(Model* m) {
     const long v = strtol(e, &end, 10);
     if (end != e && v >= 0 && v < (1l << 30)) a.spin_limit = (unsigned)v;
   }
+  // context length from which a launch uses twice the attention slices per head (WEBGPT_AMD_SHORT_KEYS for tuning)
+  a.short_keys = PD_SHORT_KEYS;
+  if (const char* e = getenv("WEBGPT_AMD_SHORT_KEYS")) {
+    char* end = nullptr;
+    const long v = strtol(e, &end, 10);
+    if (end != e && v >= 0 && v <= PD_SHORT_KEYS) a.short_keys = (int)v;
+  }
   a.trace = nullptr;
 #ifdef WGPT_TRACE
   // Profiling builds: per-workgroup clock samples of the last step of each launch.
@@ -453,7 +460,7 @@ static int decode_persistent(Model* m, int steps, int top_k = 1, double temperat
   // steps that attend to at most PD_SHORT_KEYS positions run the instantiation with half the key/value
   // registers; a run that crosses that context length is two launches, the second taking its first
   // token from the ids the first one wrote
-  const int short_steps = PD_SHORT_KEYS - m->pos;
+  const int short_steps = a.short_keys - m->pos;
   if (short_steps > 0 && short_steps < steps) {
     a.nsteps = short_steps;
     LAUNCH(launch_decode_persistent(a, rt().stream));
