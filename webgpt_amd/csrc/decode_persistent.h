@@ -58,7 +58,8 @@ struct PersistentArgs {
   // {value, epoch} exchange buffers
   unsigned long long *bufQKV, *bufATT, *bufR1, *bufH, *bufR2, *bufAM;
   float* logits;
-  const int32_t* tok;  // tok[0]: token of the first step
+  const int32_t* tok;  // tok[0]: token of the first step; null: tok_value is (a call that brings its token as an argument saves a copy)
+  int32_t tok_value;
   int32_t* out_tok;    // [nsteps] arg-max of each step
   int* err;            // set non-zero when a bounded wait expired
   unsigned long long* trace;  // optional [G][512] clock samples of the last step (WGPT_TRACE builds), or null

@@ -839,7 +839,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   typedef ItemLoader<PE, EKS ? LAY_KSPLIT : LAY_RUNS, WS, Item> LoadE;
   float4 kreg[MAXKV], vreg[MAXKV];
   unsigned ep = a.ebase;
-  int tok = a.tok[0];
+  int tok = a.tok ? a.tok[0] : a.tok_value;
 
   // the layer's block for this workgroup is already in the layout of colp (build_colparams): one load per thread
   float preg = 0.f;

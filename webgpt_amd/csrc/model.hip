@@ -389,7 +389,7 @@ static int setup_persistent(Model* m) {
   a.bufH = a.bufR1 + d;
   a.bufR2 = a.bufH + hid;
   a.bufAM = a.bufR2 + d;
-  if ((rc = dev_alloc(m, sizeof(int), (void**)&m->perr))) return rc;
+  m->perr = reinterpret_cast<int*>(m->logits + m->V);
   WGPT_HIP(hipMemsetAsync(m->perr, 0, sizeof(int), rt().stream));
   a.logits = m->logits;
   a.tok = m->tok_dev;
@@ -442,8 +442,12 @@ static int setup_persistent(Model* m) {
 // Runs `steps` greedy decode steps from position m->pos with the persistent kernel.
 // The first token is in m->tok_dev[0]; chosen ids land in m->out_tok_dev.
 // top_k == 1: greedy. Otherwise u_dev holds the steps' uniform draws.
-static int decode_persistent(Model* m, int steps, int top_k = 1, double temperature = 1.0, const double* u_dev = nullptr) {
+static int decode_persistent(Model* m, int steps, int top_k = 1, double temperature = 1.0, const double* u_dev = nullptr, int token = -1) {
   PersistentArgs a = m->pa;
+  if (token >= 0) {  // the first token travels with the launch instead of through tok_dev
+    a.tok = nullptr;
+    a.tok_value = token;
+  }
   a.top_k = top_k;
   a.temperature = temperature;
   a.u = u_dev;
@@ -505,9 +509,14 @@ static int finish_timed(Model* m, float* logits) {
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   // the logits cross the bus into pinned memory (a copy into the caller's pageable buffer is staged by the
   // runtime in pieces) and are handed over with a host copy
-  if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
-  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
+  if (logits && m->perr) {  // the error word rides behind the logits
+    WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * ((size_t)m->V + 1), hipMemcpyDeviceToHost, rt().stream));
+  } else {
+    if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+    if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
+  }
   WGPT_HIP(hipStreamSynchronize(rt().stream));
+  if (logits && m->perr) memcpy(&m->pin[1], m->logits_pin + m->V, sizeof(int));
   if (logits) memcpy(logits, m->logits_pin, sizeof(float) * (size_t)m->V);
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   return WGPT_OK;
@@ -603,12 +612,13 @@ int wgpt_model_finalize(wgpt_model h) {
   if ((rc = dev_alloc(m, T * d * f, (void**)&m->att))) return rc;
   if ((rc = dev_alloc(m, T * d * f, (void**)&m->tmp))) return rc;
   if ((rc = dev_alloc(m, T * 4 * d * f, (void**)&m->h))) return rc;
-  if ((rc = dev_alloc(m, (size_t)m->V * f, (void**)&m->logits))) return rc;
+  // the error word of the persistent kernel lives right behind the logits, so that one copy brings both back
+  if ((rc = dev_alloc(m, ((size_t)m->V + 1) * f, (void**)&m->logits))) return rc;
   if ((rc = dev_alloc(m, T * sizeof(int32_t), (void**)&m->tok_dev))) return rc;
   if (!m->pin) {
     WGPT_HIP(hipHostMalloc((void**)&m->pin, 4 * sizeof(int32_t), hipHostMallocDefault));
     m->pin[0] = m->pin[1] = m->pin[2] = m->pin[3] = 0;
-    WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * (size_t)m->V, hipHostMallocDefault));
+    WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * ((size_t)m->V + 1), hipHostMallocDefault));
   }
   if ((rc = dev_alloc(m, sizeof(int), (void**)&m->pos_dev))) return rc;
   m->att_nslice = attention_decode_slices(m->hs, m->ctx);
@@ -666,12 +676,14 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode: token id %d outside [0, %d)", token, m->V);
   if (m->pos >= m->ctx) return fail(WGPT_ERR_STATE, "wgpt_decode: context of %d positions is full; prefill a slid window", m->ctx);
-  m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
-  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   int rc;
-  if (m->decode_mode != 1 && (rc = upload_position(m))) return rc;
+  if (m->decode_mode != 1) {  // (the persistent kernel takes the token as a launch argument)
+    m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
+    WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
+    if ((rc = upload_position(m))) return rc;
+  }
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  rc = m->decode_mode == 1 ? decode_persistent(m, 1) : decode_token_blocks(m, m->pos);
+  rc = m->decode_mode == 1 ? decode_persistent(m, 1, 1, 1.0, nullptr, token) : decode_token_blocks(m, m->pos);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
@@ -689,16 +701,16 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   if (steps < 1 || !out_tokens) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: steps >= 1 and out_tokens required");
   if (m->pos + steps > m->ctx)
     return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: %d steps from position %d exceed the context of %d", steps, m->pos, m->ctx);
-  m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
-  WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
   const bool persistent = m->decode_mode == 1;
-  if (!persistent) {
+  if (!persistent) {  // (the persistent kernel takes the token as a launch argument)
+    m->pin[0] = token;  // every earlier use of the word has completed: each call ends with a synchronisation
+    WGPT_HIP(hipMemcpyAsync(m->tok_dev, &m->pin[0], sizeof(int32_t), hipMemcpyHostToDevice, rt().stream));
     int rc = upload_position(m);
     if (rc) return rc;
   }
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   if (persistent) {
-    int rc = decode_persistent(m, steps);
+    int rc = decode_persistent(m, steps, 1, 1.0, nullptr, token);
     if (rc) return rc;
   } else {
     for (int i = 0; i < steps; ++i) {
@@ -754,7 +766,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   const int pos_before = m->pos;
   int rc = WGPT_OK;
   if (in_kernel) {
-    rc = decode_persistent(m, steps, k, temperature, m->u_dev);
+    rc = decode_persistent(m, steps, k, temperature, m->u_dev, token);
   } else {
     for (int i = 0; i < steps && rc == WGPT_OK; ++i) {
       // one token per launch: the sampled id in tok_dev[0] is the next launch's input
