@@ -307,6 +307,13 @@ __device__ __forceinline__ void zero_item(float4& v) { v = make_float4(0.f, 0.f,
 __device__ __forceinline__ void zero_item(int& v) { v = 0; }
 __device__ __forceinline__ float4 to_float4(const float4& v) { return v; }
 __device__ __forceinline__ float4 to_float4(int v) { return bytes_to_float4(v); }
+// One item's contribution to a running sum. int8 items (whose phases are bound by their vector instructions: four
+// conversions per word) take four chained multiply-adds, fp32 items two products, two multiply-adds and two additions.
+template <bool CHAIN>
+__device__ __forceinline__ float item_sum(float acc, const float4& w, const float4& x) {
+  if constexpr (CHAIN) return __builtin_fmaf(w.w, x.w, __builtin_fmaf(w.z, x.z, __builtin_fmaf(w.y, x.y, __builtin_fmaf(w.x, x.x, acc))));
+  else return acc + ((w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w));
+}
 
 // f(std::integral_constant<int, i>) for i = 0 .. N-1.
 template <class F, int... Is>
@@ -603,7 +610,7 @@ __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const
       constexpr int seg = decltype(SG)::value;
       const float4 x = LNORM ? xr[LNORM ? seg : 0] : *reinterpret_cast<const float4*>(xl + seg * SEG);
       const float4 w = to_float4(ws.w[cc * P::S + seg]);
-      acc += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+      acc = item_sum<std::is_same<decltype(ws.w[0] + 0), int>::value>(acc, w, x);
     };
     if constexpr (std::is_same<R, NoRequests>::value) {
       if (valid) static_for<P::S>(item);
@@ -677,7 +684,7 @@ __device__ __forceinline__ void gemv_ksplit(const WS& ws, const float* xs, float
     static_for<P::CPW>([&](auto CI) {
       constexpr int c = decltype(CI)::value;
       const float4 w = to_float4(ws.w[si * P::CPW + c]);
-      acc[c] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+      acc[c] = item_sum<std::is_same<decltype(ws.w[0] + 0), int>::value>(acc[c], w, x);
       next.template slot<si * P::CPW + c, KSplit<P>::IPW>();
       pin_requests<R>();
     });
