@@ -57,7 +57,8 @@ struct Model {
   // [1] the error word on its way back, so that a decode call needs one stream synchronisation, [2] the cache position
   // on its way to pos_dev
   int32_t* pin = nullptr;
-  float* logits_pin = nullptr;  // pinned host copy of the logits of the last call (V floats)
+  float* logits_pin = nullptr;  // pinned host copy of the logits of the last call (V floats and the error word behind them)
+  int32_t* ids_pin = nullptr;   // pinned host copy of the ids of a multi-step call (ctx ints)
   unsigned epoch = 0;        // last epoch published by earlier launches
 
   // decode with one launch per block (decode_mode 0): the token's launches read the cache position from pos_dev and

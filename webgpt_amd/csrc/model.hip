@@ -522,6 +522,25 @@ static int finish_timed(Model* m, float* logits) {
   return WGPT_OK;
 }
 
+// The ids (and, if asked for, the logits) of a multi-step call come back through pinned memory: a copy into the caller's
+// pageable arrays is staged by the runtime and costs tens of microseconds per call. Ends with the stream drained.
+static int finish_steps(Model* m, int32_t* out_tokens, const int32_t* ids_dev, int steps, float* logits) {
+  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
+  WGPT_HIP(hipMemcpyAsync(m->ids_pin, ids_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
+  if (logits && m->perr) {  // the error word rides behind the logits
+    WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * ((size_t)m->V + 1), hipMemcpyDeviceToHost, rt().stream));
+  } else {
+    if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+    if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
+  }
+  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  memcpy(out_tokens, m->ids_pin, sizeof(int32_t) * (size_t)steps);
+  if (logits && m->perr) memcpy(&m->pin[1], m->logits_pin + m->V, sizeof(int));
+  if (logits) memcpy(logits, m->logits_pin, sizeof(float) * (size_t)m->V);
+  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  return WGPT_OK;
+}
+
 static void destroy_model(Model* m) {
   for (int v = 0; v < 2; ++v) {
     if (m->token_graph_exec[v]) (void)hipGraphExecDestroy(m->token_graph_exec[v]);
@@ -530,6 +549,7 @@ static void destroy_model(Model* m) {
   for (void* p : m->allocs) (void)hipFree(p);
   if (m->pin) (void)hipHostFree(m->pin);
   if (m->logits_pin) (void)hipHostFree(m->logits_pin);
+  if (m->ids_pin) (void)hipHostFree(m->ids_pin);
   if (m->ev0) (void)hipEventDestroy(m->ev0);
   if (m->ev1) (void)hipEventDestroy(m->ev1);
   delete m;
@@ -619,6 +639,7 @@ int wgpt_model_finalize(wgpt_model h) {
     WGPT_HIP(hipHostMalloc((void**)&m->pin, 4 * sizeof(int32_t), hipHostMallocDefault));
     m->pin[0] = m->pin[1] = m->pin[2] = m->pin[3] = 0;
     WGPT_HIP(hipHostMalloc((void**)&m->logits_pin, sizeof(float) * ((size_t)m->V + 1), hipHostMallocDefault));
+    WGPT_HIP(hipHostMalloc((void**)&m->ids_pin, sizeof(int32_t) * (size_t)m->ctx, hipHostMallocDefault));
   }
   if ((rc = dev_alloc(m, sizeof(int), (void**)&m->pos_dev))) return rc;
   m->att_nslice = attention_decode_slices(m->hs, m->ctx);
@@ -719,12 +740,10 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
       LAUNCH(launch_argmax(m->V, m->logits, m->tok_dev, m->out_tok_dev, i, rt().stream));
     }
   }
-  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
-  WGPT_HIP(hipMemcpyAsync(out_tokens, m->out_tok_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
-  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
-  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
-  WGPT_HIP(hipStreamSynchronize(rt().stream));
-  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  {
+    int rc = finish_steps(m, out_tokens, m->out_tok_dev, steps, logits);
+    if (rc) return rc;
+  }
   if (persistent) {
     int rc = check_persistent(m);
     if (rc) return rc;
@@ -783,12 +802,10 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
     (void)hipStreamSynchronize(rt().stream);
     return rc;
   }
-  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
-  WGPT_HIP(hipMemcpyAsync(out_tokens, in_kernel ? m->out_tok_dev : m->out_samp_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
-  if (logits) WGPT_HIP(hipMemcpyAsync(logits, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
-  if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
-  WGPT_HIP(hipStreamSynchronize(rt().stream));
-  WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+  if ((rc = finish_steps(m, out_tokens, in_kernel ? m->out_tok_dev : m->out_samp_dev, steps, logits))) {
+    m->pos = pos_before;
+    return rc;
+  }
   if (persistent && (rc = check_persistent(m))) return rc;
   m->pos = pos_before + steps;
   return WGPT_OK;
