@@ -365,10 +365,11 @@ def test_per_block_decode_graph_replays_equal_eager_launches(device, monkeypatch
 @pytest.mark.parametrize("graph", [False, True])
 @pytest.mark.parametrize("n_head,n_embd,n_ctx,start", [(2, 128, 600, 250), (3, 96, 1100, 1020)])
 def test_per_block_decode_across_cache_slices(device, monkeypatch, graph, n_head, n_embd, n_ctx, start):
-    """Decode mode 0 serves a context inside the first slice of the cache (256 positions at head size 64, 512 at 32)
-    with one workgroup per head and longer ones with a workgroup per (head, slice) whose results the attention
-    projection merges. Steps on both sides of the boundary, issued one by one and replayed as graphs, against the
-    oracle's full forward over the history (model.js:104-241)."""
+    """Decode mode 0 attends with a workgroup per (head, slice of the cache: 64 positions at head size 64, 128 at 32)
+    and merges the slices in the attention projection; the slices the host expects to hold positions request their
+    rows early, the others look at the position first. Steps on both sides of slice boundaries (and of the end of
+    a cache that is not a whole number of slices), issued one by one and replayed as a graph (which expects only
+    the first slice), against the oracle's full forward over the history (model.js:104-241)."""
     cfg = small_cfg(n_layer=2, n_head=n_head, n_embd=n_embd, n_ctx=n_ctx, vocab_size=97)
     if graph:
         monkeypatch.setenv("WEBGPT_AMD_TOKEN_GRAPH", "1")
@@ -379,7 +380,7 @@ def test_per_block_decode_across_cache_slices(device, monkeypatch, graph, n_head
     gpt.prefill(tokens[:start])
     for i in range(12):
         got = gpt.decode(int(tokens[start + i]))
-        if i in (0, 3, 4, 5, 6, 11):  # hs 64: 255 is the last position of the first slice; hs 32: 1024 the first of the third
+        if i in (0, 3, 4, 5, 6, 11):  # hs 64: position 256 starts a slice; hs 32: position 1024 does
             want = ref.forward(p, w, tokens[:start + i + 1])
             assert close(got, want), (i, worst(got, want))
     ids = gpt.decode_greedy(int(np.argmax(got)), 3)

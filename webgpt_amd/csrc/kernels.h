@@ -103,13 +103,14 @@ hipError_t launch_embed_at(const int32_t* tok, int d, const int* pos, const floa
 // Attention of the one query at position *pos (q[h*hs..]) over cache rows 0..*pos of a head-major cache [H][ctx][hs].
 hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc, float* out,
                                    const int* pos, hipStream_t s);
-// The same for a cache of more than one slice (attention_decode_slices(hs, ctx) > 1; a slice is 16 x 256 / lanes-per-key
-// positions, 256 at head size 64): a workgroup per (head, slice), results left in out->part for the merge of
-// launch_gemv_slab.
+// The same for a cache of more than one slice (attention_decode_slices(hs, ctx) > 1; a slice is 4 x 256 / lanes-per-key
+// positions, 64 at head size 64): a workgroup per (head, slice), results left in out->part for the merge of
+// launch_gemv_slab. spec_pos: the position the caller expects *pos to hold (slices up to it request their rows before
+// they have read *pos; any value gives the same results).
 int attention_decode_slice_positions(int hs);
 int attention_decode_slices(int hs, int ctx);
 hipError_t launch_attention_decode_slices(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc,
-                                          const AttnSlices* out, const int* pos, hipStream_t s);
+                                          const AttnSlices* out, const int* pos, int spec_pos, hipStream_t s);
 // logits[v] = LayerNorm(x) . wte[v,:], then *pos += 1: the end of a decode token.
 hipError_t launch_vocab_gemv_ln(int V, int d, const float* x, const float* gamma, const float* beta, const float* wte, float* logits,
                                 int* pos, hipStream_t s);

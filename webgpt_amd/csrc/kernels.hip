@@ -1550,17 +1550,22 @@ __global__ __launch_bounds__(WG) void attention_decode_kernel(int hs, int lpk, i
   }
 }
 
-// The same attention for caches longer than one batch (U x WG / lpk positions: 256 at head size 64): the cache is cut
-// into fixed slices of that many positions, a workgroup per (head, slice), so every slice is one memory round trip
-// whatever the context, and a long context is read by several compute units instead of one. A slice leaves
-// (sum_j e_j v_j, m, sum_j e_j) with e_j = exp(score_j - m), m its own maximum (flash-decoding); a slice beyond the
+// The same attention with the cache cut into fixed slices of ADS_ROWS x WG / lanes-per-key positions (64 at head size
+// 64), a workgroup per (head, slice): the rows of a slice are one small request per lane group, so a context of any
+// length is one memory round trip, spread over as many compute units as it has slices (one workgroup per head
+// streaming a whole context is bound by what a single compute unit can fetch: 10 us at 150 positions, 25 us at 550).
+// A slice up to the position the caller expects (spec_pos, the host's knowledge of *pos) requests its rows before it
+// has read *pos; the others read *pos first and leave at once if they lie beyond the context. A slice leaves
+// (sum_j e_j v_j, m, sum_j e_j) with e_j = exp(score_j - m), m its own maximum (flash-decoding); one beyond the
 // context leaves (0, -FLT_MAX, 0). The consumer (gemv_slab_kernel, ROW_MERGE) combines them:
 // out = sum_s w_s o_s / sum_s w_s l_s with w_s = exp(m_s - max_s m_s), which is softmax(scores) . V of
 // instructions.js:1129-1212 in another order of summation.
+constexpr int ADS_ROWS = 4;
 __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int lpk, int ctx, float scale, const float* __restrict__ q,
                                                                      const float* __restrict__ Kc, const float* __restrict__ Vc,
-                                                                     size_t hstride, float* __restrict__ part, const int* __restrict__ pos) {
-  constexpr int U = 16;
+                                                                     size_t hstride, float* __restrict__ part, const int* __restrict__ pos,
+                                                                     int spec_pos) {
+  constexpr int U = ADS_ROWS;
   extern __shared__ __attribute__((aligned(16))) float scores[];  // [U * WG / lpk]
   __shared__ float red[1024];
   __shared__ float sh[NWAVE];
@@ -1570,13 +1575,14 @@ __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int 
   const bool act = sub * 4 < hs;
   const float* kbase = Kc + h * hstride + (act ? sub * 4 : 0);
   const float* vbase = Vc + h * hstride + (act ? sub * 4 : 0);
-  // The first slice always has positions: it requests its rows before the position is known (rows up to the end of
-  // the cache exist), as attention_decode_kernel does. The others look at the position first: most of them are
-  // beyond the context most of the time, and their rows would be 3/4 of the launch's traffic for nothing.
+  // An expected slice requests its rows before the position is known (rows up to the end of the cache exist), as
+  // attention_decode_kernel does. The others look at the position first: most of them are beyond the context most of
+  // the time, and their rows would be most of the launch's traffic for nothing.
+  const bool spec = j_lo <= spec_pos;  // the caller expects this slice to have positions
   int n_here = 0;
-  if (sl > 0) n_here = min(*pos + 1 - j_lo, U * ngrp);
+  if (!spec) n_here = min(*pos + 1 - j_lo, U * ngrp);
   float* dst = part + ((size_t)h * nsl + sl) * (hs + 4);
-  if (sl > 0 && n_here <= 0) {
+  if (!spec && n_here <= 0) {
     if (tid < hs) dst[tid] = 0.f;
     if (tid == 0) {
       dst[hs] = -3.402823e+38f;
@@ -1597,7 +1603,17 @@ __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int 
     j = j < ctx ? j : ctx - 1;
     v0[u] = ld4(vbase + (size_t)j * hs);
   }
-  if (sl == 0) n_here = min(*pos + 1, U * ngrp);  // positions of this slice inside the context
+  if (spec) {
+    n_here = min(*pos + 1 - j_lo, U * ngrp);  // positions of this slice inside the context
+    if (n_here <= 0) {                        // (the caller's expectation was wrong)
+      if (tid < hs) dst[tid] = 0.f;
+      if (tid == 0) {
+        dst[hs] = -3.402823e+38f;
+        dst[hs + 1] = 0.f;
+      }
+      return;
+    }
+  }
   const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -2167,7 +2183,7 @@ hipError_t launch_attention_decode(int H, int hs, int ctx, float scale, const fl
 int attention_decode_slice_positions(int hs) {
   int lpk = 1;
   while (lpk * 4 < hs) lpk <<= 1;
-  return lpk > 64 ? 0 : 16 * (WG / lpk);
+  return lpk > 64 ? 0 : ADS_ROWS * (WG / lpk);
 }
 
 int attention_decode_slices(int hs, int ctx) {
@@ -2176,12 +2192,13 @@ int attention_decode_slices(int hs, int ctx) {
 }
 
 hipError_t launch_attention_decode_slices(int H, int hs, int ctx, float scale, const float* q, const float* Kc, const float* Vc,
-                                          const AttnSlices* out, const int* pos, hipStream_t s) {
+                                          const AttnSlices* out, const int* pos, int spec_pos, hipStream_t s) {
   int lpk = 1;
   while (lpk * 4 < hs) lpk <<= 1;
   if (lpk > 64 || hs > 256 || (hs & 3) || !out || out->hs != hs || out->nslice != attention_decode_slices(hs, ctx)) return hipErrorInvalidValue;
-  const size_t smem = sizeof(float) * 16 * (WG / lpk);
-  attention_decode_slice_kernel<<<dim3(H, out->nslice), WG, smem, s>>>(hs, lpk, ctx, scale, q, Kc, Vc, (size_t)ctx * hs, out->part, pos);
+  const size_t smem = sizeof(float) * ADS_ROWS * (WG / lpk);
+  attention_decode_slice_kernel<<<dim3(H, out->nslice), WG, smem, s>>>(hs, lpk, ctx, scale, q, Kc, Vc, (size_t)ctx * hs, out->part, pos,
+                                                                       spec_pos);
   return hipGetLastError();
 }
 

@@ -64,8 +64,8 @@ struct Model {
   // decode with one launch per block (decode_mode 0): the token's launches read the cache position from pos_dev and
   // are recorded once as a HIP graph that every later token replays
   int* pos_dev = nullptr;
-  hipGraph_t token_graph[2] = {nullptr, nullptr};          // [1]: contexts beyond the first slice of the cache
-  hipGraphExec_t token_graph_exec[2] = {nullptr, nullptr};
+  hipGraph_t token_graph = nullptr;
+  hipGraphExec_t token_graph_exec = nullptr;
   bool token_graph_tried = false;
   // attention of a decode token over a cache of more than one slice: (output, maximum, sum) per head and slice
   float* att_part = nullptr;

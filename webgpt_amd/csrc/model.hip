@@ -212,10 +212,10 @@ static int token_launches(Model* m, int pos) {
   const size_t lane_bytes = i8 ? sizeof(int32_t) : sizeof(float4);
   // fp32 slabs carry the LayerNorm gains and their biases the LayerNorm biases: the row is only normalised
   const int ln_mode = i8 ? GEMV_ROW_LAYERNORM : GEMV_ROW_NORMALISE;
-  // `pos` is what the host knows of the token's cache position; the launches themselves read it from the device. It
-  // only chooses the attention: a context that fits the first slice of the cache is served by the
-  // one-workgroup-per-head kernel, which costs a launch of H instead of H x slices workgroups and no merge.
-  const bool sliced = m->att_nslice > 1 && pos + 1 > attention_decode_slice_positions(hs);
+  // `pos` is what the host knows of the token's cache position (0 when the launches are recorded for replay); the
+  // launches themselves read it from the device. It is only a hint to the attention: the slices of the cache up to it
+  // request their rows before they have read the position, the others look first.
+  const bool sliced = m->att_nslice > 1;  // a cache of one slice is served by the one-workgroup-per-head kernel
   LAUNCH(launch_embed_at(m->tok_dev, d, m->pos_dev, m->wte, m->wpe, m->x, s));
   for (int li = 0; li < m->L; ++li) {
     const LayerW& l = m->layers[li];
@@ -228,7 +228,7 @@ static int token_launches(Model* m, int pos) {
                             m->pos_dev, s));
     if (sliced) {  // a workgroup per (head, slice of the cache), merged as c_proj stages its row
       const AttnSlices sl = {m->att_part, m->att_nslice, hs};
-      LAUNCH(launch_attention_decode_slices(H, hs, m->ctx, scale, m->qkv, Kc, Vc, &sl, m->pos_dev, s));
+      LAUNCH(launch_attention_decode_slices(H, hs, m->ctx, scale, m->qkv, Kc, Vc, &sl, m->pos_dev, pos, s));
       LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, nullptr, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
                               EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s, &sl));
     } else {
@@ -265,38 +265,25 @@ static int decode_token_blocks(Model* m, int pos) {
     const char* on = getenv("WEBGPT_AMD_TOKEN_GRAPH");
     if (on && on[0] == '1') {
       WGPT_HIP(hipStreamSynchronize(s));
-      // One graph per attention variant (the context inside the first slice of the cache, or beyond it), so that a
-      // replay runs exactly the launches the host would issue. A recording run changes nothing on the device.
-      const int variants = m->att_nslice > 1 ? 2 : 1;
-      bool ok = true;
-      for (int v = 0; v < variants && ok; ++v) {
-        ok = false;
-        if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
-          const int rc = token_launches(m, v == 0 ? 0 : m->ctx - 1);
-          hipGraph_t g = nullptr;
-          const hipError_t e = hipStreamEndCapture(s, &g);
-          if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec[v], g, nullptr, nullptr, 0) == hipSuccess) {
-            m->token_graph[v] = g;
-            ok = true;
-          } else if (g) {
-            (void)hipGraphDestroy(g);
-          }
+      // a recording run changes nothing on the device: what is recorded is replayed below
+      if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        const int rc = token_launches(m, 0);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(s, &g);
+        if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
+          m->token_graph = g;
+        } else {
+          if (g) (void)hipGraphDestroy(g);
+          m->token_graph_exec = nullptr;
+          (void)hipGetLastError();
         }
-      }
-      if (!ok) {  // issue the launches instead
-        for (int v = 0; v < 2; ++v) {
-          if (m->token_graph_exec[v]) (void)hipGraphExecDestroy(m->token_graph_exec[v]);
-          if (m->token_graph[v]) (void)hipGraphDestroy(m->token_graph[v]);
-          m->token_graph_exec[v] = nullptr;
-          m->token_graph[v] = nullptr;
-        }
+      } else {
         (void)hipGetLastError();
       }
     }
   }
-  if (m->token_graph_exec[0]) {
-    const bool sliced = m->att_nslice > 1 && pos + 1 > attention_decode_slice_positions(m->hs);
-    WGPT_HIP(hipGraphLaunch(m->token_graph_exec[sliced ? 1 : 0], s));
+  if (m->token_graph_exec) {
+    WGPT_HIP(hipGraphLaunch(m->token_graph_exec, s));
     return WGPT_OK;
   }
   return token_launches(m, pos);
@@ -542,10 +529,8 @@ static int finish_steps(Model* m, int32_t* out_tokens, const int32_t* ids_dev, i
 }
 
 static void destroy_model(Model* m) {
-  for (int v = 0; v < 2; ++v) {
-    if (m->token_graph_exec[v]) (void)hipGraphExecDestroy(m->token_graph_exec[v]);
-    if (m->token_graph[v]) (void)hipGraphDestroy(m->token_graph[v]);
-  }
+  if (m->token_graph_exec) (void)hipGraphExecDestroy(m->token_graph_exec);
+  if (m->token_graph) (void)hipGraphDestroy(m->token_graph);
   for (void* p : m->allocs) (void)hipFree(p);
   if (m->pin) (void)hipHostFree(m->pin);
   if (m->logits_pin) (void)hipHostFree(m->logits_pin);
