@@ -94,6 +94,7 @@ enum { GEMV_ROW_PLAIN = 0, GEMV_ROW_NORMALISE = 1, GEMV_ROW_LAYERNORM = 2 };
 struct AttnSlices {
   float* part;  // [H][nslice][hs + 4]: unnormalised output, then the slice's maximum and sum
   int nslice, hs;
+  int nmerge;   // the merge reads the first nmerge slices: at least those that hold positions (nslice is always right)
 };
 hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const float* scale, const float* x, int row_mode,
                             const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,

@@ -1291,8 +1291,9 @@ struct GemvSlabArgs {
   float* Vc;
   int d, hs, ctx;
   const int* pos;
-  int nslice;           // ROW_MERGE: x holds [K / mhs][nslice][mhs + 4] attention slices
+  int nslice;           // ROW_MERGE: x holds [K / mhs][nslice][mhs + 4] attention slices, of which the first nmerge are read
   int mhs;
+  int nmerge;
 };
 
 typedef float nt_f32x4 __attribute__((ext_vector_type(4)));
@@ -1351,12 +1352,12 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
         const float* ph = a.x + (size_t)h * a.nslice * stride;
         // eight slices at a time, everything requested before anything is used: one round trip, not one per slice
         float mx = -3.402823e+38f, den = 0.f;
-        for (int s0 = 0; s0 < a.nslice; s0 += 8) {
+        for (int s0 = 0; s0 < a.nmerge; s0 += 8) {
           float mv[8], lv[8];
           float4 ov[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            const int sl = s0 + j < a.nslice ? s0 + j : a.nslice - 1;
+            const int sl = s0 + j < a.nmerge ? s0 + j : a.nmerge - 1;
             mv[j] = ph[sl * stride + a.mhs];
             lv[j] = ph[sl * stride + a.mhs + 1];
             ov[j] = ld4(ph + sl * stride + e);
@@ -1364,14 +1365,14 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
           float mnew = mx;
 #pragma unroll
           for (int j = 0; j < 8; ++j)
-            if (s0 + j < a.nslice) mnew = fmaxf(mnew, mv[j]);
+            if (s0 + j < a.nmerge) mnew = fmaxf(mnew, mv[j]);
           const float keep = expf(mx - mnew);  // rescales what earlier groups of eight have left
           den *= keep;
           v = make_float4(v.x * keep, v.y * keep, v.z * keep, v.w * keep);
           mx = mnew;
 #pragma unroll
           for (int j = 0; j < 8; ++j)
-            if (s0 + j < a.nslice) {
+            if (s0 + j < a.nmerge) {
               const float w = expf(mv[j] - mx);
               den += w * lv[j];
               fma4(v, w, ov[j]);
@@ -2147,13 +2148,15 @@ hipError_t launch_gemv_slab(int N, int K, const void* slab, bool int8, const flo
                             const float* gamma, const float* beta, const float* bias, float* C, int epi, const float* resid,
                             const KvAfter* kv, const int* pos, hipStream_t s, const AttnSlices* merge) {
   if ((K & 3) || N < 1) return hipErrorInvalidValue;
-  if (merge && (row_mode != GEMV_ROW_PLAIN || merge->nslice < 1 || merge->hs < 4 || (merge->hs & 3) || K % merge->hs)) return hipErrorInvalidValue;
+  if (merge && (row_mode != GEMV_ROW_PLAIN || merge->nslice < 1 || merge->nmerge < 1 || merge->nmerge > merge->nslice || merge->hs < 4 ||
+                (merge->hs & 3) || K % merge->hs))
+    return hipErrorInvalidValue;
   const int S = cdiv(K, 256);
   const size_t lds = sizeof(float) * (size_t)S * 256;
   if (lds > 48 * 1024) return hipErrorInvalidValue;
   GemvSlabArgs a{N, K, S, slab, scale, merge ? merge->part : x, merge ? (int)ROW_MERGE : row_mode, gamma, beta, bias, epi, resid, C,
                  kv ? kv->Kc : nullptr, kv ? kv->Vc : nullptr, kv ? kv->d : 0, kv ? kv->hs : 1, kv ? kv->ctx : 0, pos,
-                 merge ? merge->nslice : 0, merge ? merge->hs : 1};
+                 merge ? merge->nslice : 0, merge ? merge->hs : 1, merge ? merge->nmerge : 0};
   if (int8) {
     if (N >= 4096) gemv_slab_kernel<4, true><<<cdiv(N, NWAVE * 4), WG, lds, s>>>(a);
     else gemv_slab_kernel<2, true><<<cdiv(N, NWAVE * 2), WG, lds, s>>>(a);

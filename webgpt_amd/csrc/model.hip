@@ -2,6 +2,7 @@
 // wgpt_model_create / set_tensor / finalize, GPT.run (model.js:104-268) becomes
 // wgpt_prefill (whole window) and wgpt_decode (window extended by one token, served
 // from a device-resident KV cache).
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -202,7 +203,7 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
 // (+ residual), c_fc (LayerNorm in, GELU out), mlp c_proj (+ residual); the final LayerNorm with the
 // vocabulary projection of that row (instructions.js:849-856), which also advances the position. 5L + 2 launches, none of
 // which carries the position as an argument. The products read the decode slabs (a column's K values contiguous).
-static int token_launches(Model* m, int pos) {
+static int token_launches(Model* m, int pos, bool recording = false) {
   hipStream_t s = rt().stream;
   const int d = m->d, H = m->H, hs = m->hs, hid = 4 * d;
   const float scale = (float)(1.0 / std::sqrt((double)hs));  // model.js:321
@@ -227,7 +228,9 @@ static int token_launches(Model* m, int pos) {
     LAUNCH(launch_gemv_slab(3 * d, d, slab, i8, lp + po.sA, m->x, ln_mode, l.ln1_g, l.ln1_b, lp + po.bA, m->qkv, EPI_NONE, nullptr, &kva,
                             m->pos_dev, s));
     if (sliced) {  // a workgroup per (head, slice of the cache), merged as c_proj stages its row
-      const AttnSlices sl = {m->att_part, m->att_nslice, hs};
+      // (a recorded token merges all slices: those beyond the context hold zeros with weight zero)
+      const int per = attention_decode_slice_positions(hs);
+      const AttnSlices sl = {m->att_part, m->att_nslice, hs, recording ? m->att_nslice : std::min(m->att_nslice, pos / per + 1)};
       LAUNCH(launch_attention_decode_slices(H, hs, m->ctx, scale, m->qkv, Kc, Vc, &sl, m->pos_dev, pos, s));
       LAUNCH(launch_gemv_slab(d, d, slab + a.slab_offC * lane_bytes, i8, lp + po.sC, nullptr, GEMV_ROW_PLAIN, nullptr, nullptr, lp + po.bC, m->x,
                               EPI_RESIDUAL, m->x, nullptr, m->pos_dev, s, &sl));
@@ -267,7 +270,7 @@ static int decode_token_blocks(Model* m, int pos) {
       WGPT_HIP(hipStreamSynchronize(s));
       // a recording run changes nothing on the device: what is recorded is replayed below
       if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
-        const int rc = token_launches(m, 0);
+        const int rc = token_launches(m, 0, true);
         hipGraph_t g = nullptr;
         const hipError_t e = hipStreamEndCapture(s, &g);
         if (rc == WGPT_OK && e == hipSuccess && g && hipGraphInstantiate(&m->token_graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
