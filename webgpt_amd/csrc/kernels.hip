@@ -1326,6 +1326,28 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
       sc[r] = make_float4(s, s, s, s);
     }
   }
+  // What the epilogue adds is requested now as well: a load behind the dot products would be one more memory round
+  // trip at the end of a kernel that consists of little else. (resid may be C itself: column n is read and written
+  // by its owner only.)
+  float ebias[R], eres[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int col = col0 + r < a.N ? col0 + r : a.N - 1;
+    ebias[r] = a.bias ? a.bias[col] : 0.f;
+    eres[r] = a.epi == EPI_RESIDUAL ? a.resid[col] : 0.f;
+  }
+  const int kvpos = a.Kc ? *a.pos : 0;
+  // ... and the LayerNorm parameters of this thread's first two float4 of the row (int8 slabs do not carry them)
+  float4 gpre[2], bpre[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    gpre[p] = bpre[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (a.row_mode == ROW_LAYERNORM) {
+      const int i = tid + WG * p < k4 ? tid + WG * p : k4 - 1;
+      gpre[p] = ld4(a.gamma + 4 * i);
+      bpre[p] = ld4(a.beta + 4 * i);
+    }
+  }
   Item w0[R][CH], w1[R][CH];
   auto request = [&](Item (&w)[R][CH], int c0) {
 #pragma unroll
@@ -1399,11 +1421,12 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
     }
     const float var = block_sum(q, sh) / (float)a.K;
     const float stdev = sqrtf(var + 1e-5f);
-    for (int i = tid; i < k4; i += WG) {
+    for (int i = tid, p = 0; i < k4; i += WG, ++p) {
       const float4 v = ld4(xs + 4 * i);
       float4 o = make_float4((v.x - mean) / stdev, (v.y - mean) / stdev, (v.z - mean) / stdev, (v.w - mean) / stdev);
       if (a.row_mode == ROW_LAYERNORM) {
-        const float4 g = ld4(a.gamma + 4 * i), b = ld4(a.beta + 4 * i);
+        const float4 g = p == 0 ? gpre[0] : (p == 1 ? gpre[1] : ld4(a.gamma + 4 * i));
+        const float4 b = p == 0 ? bpre[0] : (p == 1 ? bpre[1] : ld4(a.beta + 4 * i));
         o = make_float4(g.x * o.x + b.x, g.y * o.y + b.y, g.z * o.z + b.z, g.w * o.w + b.w);
       }
       st4(xs + 4 * i, o);
@@ -1440,13 +1463,13 @@ __global__ __launch_bounds__(WG) void gemv_slab_kernel(GemvSlabArgs a) {
     float v = wave_sum(acc[r]);
     const int n = col0 + r;
     if (lane == 0 && n < a.N) {
-      if (a.bias) v += a.bias[n];
+      if (a.bias) v += ebias[r];
       if (a.epi == EPI_GELU) v = gelu_ref(v);
-      else if (a.epi == EPI_RESIDUAL) v += a.resid[n];
+      else if (a.epi == EPI_RESIDUAL) v += eres[r];
       a.C[n] = v;
       if (a.Kc && n >= a.d) {
         const int which = n >= 2 * a.d, c = n - (1 + which) * a.d, h = c / a.hs, e = c - h * a.hs;
-        (which ? a.Vc : a.Kc)[((size_t)h * a.ctx + *a.pos) * a.hs + e] = v;
+        (which ? a.Vc : a.Kc)[((size_t)h * a.ctx + kvpos) * a.hs + e] = v;
       }
     }
   }
@@ -1471,6 +1494,7 @@ __global__ __launch_bounds__(WG) void attention_decode_kernel(int hs, int lpk, i
   const float* vbase = Vc + h * hstride + (act ? sub * 4 : 0);
   // The first batch is requested before the position is known (rows up to the end of the cache exist; those
   // beyond the context hold finite leftovers and are not used): its round trip overlaps that of *pos.
+  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
   float4 k0[U], v0[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -1485,7 +1509,6 @@ __global__ __launch_bounds__(WG) void attention_decode_kernel(int hs, int lpk, i
     v0[u] = ld4(vbase + (size_t)j * hs);
   }
   const int nkeys = *pos + 1;
-  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int j = u * ngrp + grp;
@@ -1579,6 +1602,7 @@ __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int 
   // An expected slice requests its rows before the position is known (rows up to the end of the cache exist), as
   // attention_decode_kernel does. The others look at the position first: most of them are beyond the context most of
   // the time, and their rows would be most of the launch's traffic for nothing.
+  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);  // (first: nothing below may wait for it)
   const bool spec = j_lo <= spec_pos;  // the caller expects this slice to have positions
   int n_here = 0;
   if (!spec) n_here = min(*pos + 1 - j_lo, U * ngrp);
@@ -1615,7 +1639,6 @@ __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int 
       return;
     }
   }
-  const float4 qv = act ? ld4(q + h * hs + sub * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int jl = u * ngrp + grp;
@@ -1665,6 +1688,22 @@ __global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const f
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int v0 = (blockIdx.x * NWAVE + wave) * VOCAB_ROWS_PER_WAVE;
   const int n4 = d >> 2;
+  // Everything that does not depend on the row is requested first, so that it travels during the LayerNorm: the first
+  // two sweeps of this wave's table rows, and the LayerNorm parameters of this thread's first two float4 of the row.
+  constexpr int PRE = 2;
+  float4 wpre[PRE][VOCAB_ROWS_PER_WAVE], gpre[PRE], bpre[PRE];
+#pragma unroll
+  for (int p = 0; p < PRE; ++p) {
+    const int c = lane + 64 * p < n4 ? lane + 64 * p : n4 - 1;
+#pragma unroll
+    for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+      const int row = v0 + r < V ? v0 + r : V - 1;
+      wpre[p][r] = ld4(wte + (size_t)row * d + 4 * c);
+    }
+    const int ct = (int)threadIdx.x + WG * p < n4 ? (int)threadIdx.x + WG * p : n4 - 1;
+    gpre[p] = ld4(gamma + 4 * ct);
+    bpre[p] = ld4(beta + 4 * ct);
+  }
   float s1 = 0.f;
   for (int c = threadIdx.x; c < n4; c += WG) {
     const float4 v = ld4(x + 4 * c);
@@ -1680,8 +1719,10 @@ __global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const f
   }
   const float var = block_sum(q, sh) / (float)d;
   const float stdev = sqrtf(var + 1e-5f);
-  for (int c = threadIdx.x; c < n4; c += WG) {
-    const float4 v = ld4(xs + 4 * c), g = ld4(gamma + 4 * c), b = ld4(beta + 4 * c);
+  for (int c = threadIdx.x, p = 0; c < n4; c += WG, ++p) {
+    const float4 v = ld4(xs + 4 * c);
+    const float4 g = p == 0 ? gpre[0] : (p == 1 ? gpre[1] : ld4(gamma + 4 * c));
+    const float4 b = p == 0 ? bpre[0] : (p == 1 ? bpre[1] : ld4(beta + 4 * c));
     st4(xs + 4 * c, make_float4(g.x * ((v.x - mean) / stdev) + b.x, g.y * ((v.y - mean) / stdev) + b.y,
                                 g.z * ((v.z - mean) / stdev) + b.z, g.w * ((v.w - mean) / stdev) + b.w));
   }
@@ -1689,7 +1730,19 @@ __global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const f
   float acc[VOCAB_ROWS_PER_WAVE];
 #pragma unroll
   for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) acc[r] = 0.f;
-  for (int c = lane; c < n4; c += 64) {
+#pragma unroll
+  for (int p = 0; p < PRE; ++p) {
+    const int c = lane + 64 * p;
+    if (c < n4) {
+      const float4 xv = ld4(xs + 4 * c);
+#pragma unroll
+      for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
+        const float4 w = wpre[p][r];
+        if (v0 + r < V) acc[r] += (xv.x * w.x + xv.y * w.y) + (xv.z * w.z + xv.w * w.w);
+      }
+    }
+  }
+  for (int c = lane + 64 * PRE; c < n4; c += 64) {
     const float4 xv = ld4(xs + 4 * c);
 #pragma unroll
     for (int r = 0; r < VOCAB_ROWS_PER_WAVE; ++r) {
