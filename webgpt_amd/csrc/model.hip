@@ -390,9 +390,9 @@ static int setup_persistent(Model* m) {
     // curves are flat within a few percent around them and over context length);
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
     static const int tuned[5][7] = {{16, 0, 20, 96, 20, 28, 48},    // d <= 768
-                                    {32, 0, 48, 96, 40, 32, 64},    // d = 1024
-                                    {16, 0, 48, 96, 4, 20, 40},     // d = 1280
-                                    {12, 12, 28, 96, 20, 12, 12},   // d = 1600, int8
+                                    {40, 0, 40, 96, 48, 40, 16},    // d = 1024
+                                    {20, 0, 40, 128, 24, 20, 40},   // d = 1280
+                                    {16, 12, 20, 112, 20, 12, 4},   // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
