@@ -209,14 +209,18 @@ __global__ __launch_bounds__(WG) void reduce_ln_kernel(int M, int N, int S, cons
                                                         const float* __restrict__ beta, float* __restrict__ ln_out, int ldo) {
   __shared__ float sh[NWAVE];
   const int r = blockIdx.x, n4 = N >> 2;
-  float4 v[REDUCE_LN_MAXV];
+  float4 v[REDUCE_LN_MAXV], gpre[REDUCE_LN_MAXV], bpre[REDUCE_LN_MAXV];
   float sum = 0.f;
 #pragma unroll
   for (int j = 0; j < REDUCE_LN_MAXV; ++j) {
     const int i = threadIdx.x + j * WG;
     v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    gpre[j] = bpre[j] = v[j];
     if (i < n4) {
       const int n0 = 4 * i;
+      // (requested with the partial sums: behind the two reductions they would be a memory round trip of their own)
+      gpre[j] = ld4(gamma + n0);
+      bpre[j] = ld4(beta + n0);
       float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
       for (int sp = 0; sp < S; ++sp) {
         const float4 p = ld4(part + ((size_t)sp * M + r) * N + n0);
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(WG) void reduce_ln_kernel(int M, int N, int S, cons
   for (int j = 0; j < REDUCE_LN_MAXV; ++j) {
     const int i = threadIdx.x + j * WG;
     if (i < n4) {
-      const float4 g = ld4(gamma + 4 * i), b = ld4(beta + 4 * i);
+      const float4 g = gpre[j], b = bpre[j];
       float4 o;
       o.x = g.x * ((v[j].x - mean) / stdev) + b.x;
       o.y = g.y * ((v[j].y - mean) / stdev) + b.y;
