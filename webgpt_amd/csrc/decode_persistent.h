@@ -17,6 +17,7 @@ constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
 constexpr int PD_COLP = 256;     // floats of one workgroup's column parameters of a layer (4 phases x 32 columns x {bias, scale})
 constexpr int PD_KVBATCH = 4;    // key batches (of 32) a slice holds in registers: n_ctx <= 32*PD_KVBATCH*PD_SPLIT_LONG
 constexpr int PD_SHORT_KEYS = 32 * PD_KVBATCH * PD_SPLIT;  // longest context of the instantiation with PD_SPLIT slices
+constexpr int PD_TABLE_LDS_STEPS = 2;  // launches of at least this many steps keep part of the vocabulary table in LDS
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
 // [w*cpw, (w+1)*cpw) of N; a column is S segments ("items") of 256 contraction elements,

@@ -854,6 +854,36 @@ struct Phases {
 
 // SAMPLE: top-k selection and sampling in the kernel (top_k in 2..PD_TOPK); the arg-max kernel
 // stays free of its registers.
+// Floats of dynamic LDS the phases use (rows, staged exchange words, partial sums, parameter blocks), rounded to
+// a multiple of four so that what follows is 16-byte aligned.
+template <class C>
+constexpr int lds_floats() {
+  typedef Phases<C> PS;
+  constexpr int XS = (C::SD + C::SH) * SEG;
+  constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;
+  constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
+  return (XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + PD_COLP + 16 + 3) / 4 * 4;
+}
+// Rows of the vocabulary table a workgroup keeps in the LDS its phases leave free, for the whole launch: the
+// first rows of its run, a multiple of the wave count, at most one batch of the vocabulary loop. A compute unit
+// has 160 KB; 2 KB stay aside for the static part.
+constexpr int PD_VOCAB_BATCH = 4;  // rows of wte in flight per wave
+template <class C>
+constexpr int table_rows_in_lds() {
+  constexpr int spare = (160 * 1024 - 2048) / 4 - lds_floats<C>();
+  // the wider shapes sit at the register limit, lose more to the extra code than the few rows that fit would give
+  // them (d = 1280: 0.784 against 0.779 ms/token, int8 d = 1600: 1.00 against 0.80), and keep none
+  constexpr int rows = (spare > 0 && C::D <= 1024 && !C::I8) ? spare / C::D / NW * NW : 0;
+  return rows > NW * PD_VOCAB_BATCH ? NW * PD_VOCAB_BATCH : rows;
+}
+
+// Rows per wave that stay in registers next to them (12 registers a row at d = 768; with the candidate lists of
+// top-k sampling a fourth row would spill).
+template <class C, bool SAMPLE>
+constexpr int table_rows_in_registers() {
+  return (table_rows_in_lds<C>() > 0 && C::D <= 768) ? (SAMPLE ? 3 : 4) : 0;
+}
+
 template <class C, int MAXKV, bool SAMPLE>
 __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a) {
   typedef Phases<C> PS;
@@ -889,6 +919,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   float* pubD = pubC + PC::CPW;   // [PD::CPW] finished c_fc columns
   float* colp = pubD + PD::CPW + PE::CPW;   // [8 * LPW] biases and int8 column scales of this workgroup's columns of the layer
   static_assert(PA::CPW <= LPW && PC::CPW <= LPW && PD::CPW <= LPW && PE::CPW <= LPW, "a phase has more columns per workgroup than colp holds");
+  // Launches of several steps keep the first LROWS rows of the workgroup's run of the vocabulary table here
+  // from start to end: that share of the table is read from memory once per launch instead of once per token.
+  constexpr int LROWS = table_rows_in_lds<C>(), LR = LROWS / NW;
+  float* vres = lds + lds_floats<C>();  // [LROWS * D]
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: same for the whole wave
@@ -942,6 +976,35 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     const int t = opaque(tid);
     if (t < PD_COLP) colp[t] = preg;
   };
+  // (not for a table so small that these rows would be most of the run: loading them then costs more than it saves)
+  const int lrows = (LROWS > 0 && a.nsteps >= PD_TABLE_LDS_STEPS && a.rows_per_wg >= 4 * LROWS) ? LROWS : 0;
+  if (lrows) {
+    const int v0 = wg * a.rows_per_wg;
+    for (int e = tid; e < LROWS * (D / 4); e += NT) {
+      const int r = e / (D / 4), c = e - r * (D / 4);
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (r < a.rows_per_wg && v0 + r < a.V) v = reinterpret_cast<const float4*>(a.wte + (size_t)(v0 + r) * D)[c];
+      reinterpret_cast<float4*>(vres)[e] = v;
+    }
+  }
+  // ... and the RROWS rows behind them in registers the narrow shapes leave free, RR per wave
+  constexpr int RR = table_rows_in_registers<C, SAMPLE>(), RROWS = RR * NW;
+  [[maybe_unused]] float4 wres[RR > 0 ? RR : 1][C::SD];
+  if constexpr (RR > 0) {
+    if (lrows) {
+      const int ln = opaque(tid & 63);
+      const int vb = wg * a.rows_per_wg + LROWS + wave * RR;
+#pragma unroll
+      for (int r = 0; r < RR; ++r)
+#pragma unroll
+        for (int s2 = 0; s2 < C::SD; ++s2) {
+          wres[r][s2] = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (LROWS + wave * RR + r < a.rows_per_wg && vb + r < a.V && (s2 * SEG + SEG <= D || s2 * SEG + ln * 4 < D))
+            wres[r][s2] = *reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * D + s2 * SEG + ln * 4);
+        }
+    }
+  }
+  const int rrows = (RR > 0 && lrows) ? RROWS : 0;
   request_params(0);
   LoadA(wX, slabs, ncA, wg, wave, lane).all();
   deposit_params();
@@ -1316,7 +1379,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     wait_loads();
     TRACE(1 + a.L * 8);
     {
-      constexpr int S = C::SD, R = 4;  // rows of wte in flight per wave
+      constexpr int S = C::SD, R = PD_VOCAB_BATCH;  // rows of wte in flight per wave
       // A table of up to 160 MB is read with ordinary loads, so that it may stay in the 256 MB memory-side cache
       // from one token to the next while the layers' weights stream past it with non-temporal loads (117M, 154 MB:
       // 0.1574 -> 0.1545 ms/token); a larger one would only push itself out (345M, 206 MB: 0.400 -> 0.425 with
@@ -1341,49 +1404,132 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         tv[j] = -INFINITY;
         ti[j] = NOCAND;
       }
-      for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
-        float4 w[R][S];
+      if constexpr (LROWS == 0) {
+        // the shapes at the register limit keep this loop exactly as it was tuned: sharing the per-row code below
+        // with them moved d = 1280 from 0.779 to 0.785 ms/token
+        for (int vb = v0 + wave * R; vb < v1; vb += NW * R) {
+          float4 w[R][S];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+          for (int r = 0; r < R; ++r)
 #pragma unroll
-          for (int s2 = 0; s2 < S; ++s2) {
-            w[r][s2] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (vb + r < v1 && (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D))
-              w[r][s2] = ld_table<WTE_RESIDENT>(reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * D + s2 * SEG + lane * 4));
-          }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          float acc = 0.f;
-#pragma unroll
-          for (int s2 = 0; s2 < S; ++s2)
-            acc += (w[r][s2].x * xv[s2].x + w[r][s2].y * xv[s2].y) + (w[r][s2].z * xv[s2].z + w[r][s2].w * xv[s2].w);
-          const float s = wave_sum(acc);
-          if (vb + r < v1) {
-            if (lane == 0) a.logits[vb + r] = s;
-            if (s > best || besti == 0x7fffffff) {
-              best = s;
-              besti = vb + r;
+            for (int s2 = 0; s2 < S; ++s2) {
+              w[r][s2] = make_float4(0.f, 0.f, 0.f, 0.f);
+              if (vb + r < v1 && (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D))
+                w[r][s2] = ld_table<WTE_RESIDENT>(reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * D + s2 * SEG + lane * 4));
             }
-            if (SAMPLE && cand_before(s, vb + r, lastv, lasti)) {
-              // insert: carry the displaced candidate down the list
-              float cv = s;
-              int ci = vb + r;
 #pragma unroll
-              for (int j = 0; j < KL; ++j) {
-                if (j < K && cand_before(cv, ci, tv[j], ti[j])) {
-                  const float sv = tv[j];
-                  const int si = ti[j];
-                  tv[j] = cv;
-                  ti[j] = ci;
-                  cv = sv;
-                  ci = si;
-                }
-                if (j == K - 1) {
-                  lastv = tv[j];
-                  lasti = ti[j];
+          for (int r = 0; r < R; ++r) {
+            float acc = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < S; ++s2)
+              acc += (w[r][s2].x * xv[s2].x + w[r][s2].y * xv[s2].y) + (w[r][s2].z * xv[s2].z + w[r][s2].w * xv[s2].w);
+            const float s = wave_sum(acc);
+            if (vb + r < v1) {
+              if (lane == 0) a.logits[vb + r] = s;
+              if (s > best || besti == 0x7fffffff) {
+                best = s;
+                besti = vb + r;
+              }
+              if (SAMPLE && cand_before(s, vb + r, lastv, lasti)) {
+                // insert: carry the displaced candidate down the list
+                float cv = s;
+                int ci = vb + r;
+#pragma unroll
+                for (int j = 0; j < KL; ++j) {
+                  if (j < K && cand_before(cv, ci, tv[j], ti[j])) {
+                    const float sv = tv[j];
+                    const int si = ti[j];
+                    tv[j] = cv;
+                    ti[j] = ci;
+                    cv = sv;
+                    ci = si;
+                  }
+                  if (j == K - 1) {
+                    lastv = tv[j];
+                    lasti = ti[j];
+                  }
                 }
               }
             }
+          }
+        }
+      } else {
+        // one finished row: logit, running arg-max (rows come in ascending order per wave: the first index wins a
+        // tie), top-k candidates
+        auto tally = [&](float s, int row) {
+          if (lane == 0) a.logits[row] = s;
+          if (s > best || besti == 0x7fffffff) {
+            best = s;
+            besti = row;
+          }
+          if (SAMPLE && cand_before(s, row, lastv, lasti)) {
+            // insert: carry the displaced candidate down the list
+            float cv = s;
+            int ci = row;
+#pragma unroll
+            for (int j = 0; j < KL; ++j) {
+              if (j < K && cand_before(cv, ci, tv[j], ti[j])) {
+                const float sv = tv[j];
+                const int si = ti[j];
+                tv[j] = cv;
+                ti[j] = ci;
+                cv = sv;
+                ci = si;
+              }
+              if (j == K - 1) {
+                lastv = tv[j];
+                lasti = ti[j];
+              }
+            }
+          }
+        };
+        if constexpr (LROWS > 0) {
+          if (lrows) {  // the lowest rows of the run, from LDS
+#pragma unroll
+            for (int r = 0; r < LR; ++r) {
+              float acc = 0.f;
+#pragma unroll
+              for (int s2 = 0; s2 < S; ++s2)
+                if (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D) {
+                  const float4 wl = *reinterpret_cast<const float4*>(vres + (wave * LR + r) * D + s2 * SEG + lane * 4);
+                  acc += (wl.x * xv[s2].x + wl.y * xv[s2].y) + (wl.z * xv[s2].z + wl.w * xv[s2].w);
+                }
+              const float s = wave_sum(acc);
+              if (v0 + wave * LR + r < v1) tally(s, v0 + wave * LR + r);
+            }
+          }
+        }
+        if constexpr (RR > 0) {
+          if (rrows) {  // the next rows, from registers
+#pragma unroll
+            for (int r = 0; r < RR; ++r) {
+              float acc = 0.f;
+#pragma unroll
+              for (int s2 = 0; s2 < S; ++s2)
+                acc += (wres[r][s2].x * xv[s2].x + wres[r][s2].y * xv[s2].y) + (wres[r][s2].z * xv[s2].z + wres[r][s2].w * xv[s2].w);
+              const float s = wave_sum(acc);
+              if (v0 + LROWS + wave * RR + r < v1) tally(s, v0 + LROWS + wave * RR + r);
+            }
+          }
+        }
+        for (int vb = v0 + lrows + rrows + wave * R; vb < v1; vb += NW * R) {
+          float4 w[R][S];
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int s2 = 0; s2 < S; ++s2) {
+              w[r][s2] = make_float4(0.f, 0.f, 0.f, 0.f);
+              if (vb + r < v1 && (s2 * SEG + SEG <= D || s2 * SEG + lane * 4 < D))
+                w[r][s2] = ld_table<WTE_RESIDENT>(reinterpret_cast<const float4*>(a.wte + (size_t)(vb + r) * D + s2 * SEG + lane * 4));
+            }
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            float acc = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < S; ++s2)
+              acc += (w[r][s2].x * xv[s2].x + w[r][s2].y * xv[s2].y) + (w[r][s2].z * xv[s2].z + w[r][s2].w * xv[s2].w);
+            const float s = wave_sum(acc);
+            if (vb + r < v1) tally(s, vb + r);
           }
         }
       }
@@ -1634,11 +1780,7 @@ __global__ void build_colparams_kernel(const float* __restrict__ lparams, int L,
 
 template <class C>
 size_t lds_bytes_of() {
-  typedef Phases<C> PS;
-  constexpr int XS = (C::SD + C::SH) * SEG;
-  constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;
-  constexpr int PART = 32 * (C::HS + 4) > PS::E::CPW * NW ? 32 * (C::HS + 4) : PS::E::CPW * NW;
-  const size_t need = sizeof(float) * (size_t)(XS + 2 * C::D + ATTP + PART + 3 * C::HS + PS::A::CPW + 2 * PS::Cc::CPW + PS::Dd::CPW + PD_COLP + 16);
+  const size_t need = sizeof(float) * (size_t)(lds_floats<C>() + table_rows_in_lds<C>() * C::D);
   // more than half of a compute unit's 160 KB, so that exactly one workgroup lives on each
   const size_t one_per_cu = 84 * 1024;
   return need > one_per_cu ? need : one_per_cu;
