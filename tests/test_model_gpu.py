@@ -224,6 +224,29 @@ def test_larger_shapes_decode_against_oracle(device, name):
     gpt.unloadBuffers()
 
 
+@pytest.mark.parametrize("name,n_layer", [("gpt2-117m", 2), ("gpt2-345m", 2)])
+def test_multi_step_launch_logits_equal_single_step_launches(device, name, n_layer):
+    # A launch of several steps keeps part of the vocabulary table on the chip (LDS, registers) and reads the rest
+    # from memory; a single-step launch reads all of it from memory. Same sums, same order: the logits of the last
+    # step are the same bits, and so is every chosen token (full 50257-row table, so every workgroup has a full run).
+    cfg = dict(synth.CONFIGS[name])
+    cfg["n_layer"] = n_layer
+    gpt, _ = load(cfg, seed=21, random_ln=True)
+    gpt.set_decode_mode(1)
+    tokens = synth.tokens(5, "prompt", 40, cfg["vocab_size"])
+    first = int(np.argmax(gpt.prefill(tokens)))
+    ids, last = gpt.decode_greedy(first, 6, want_logits=True)
+    gpt.prefill(tokens)
+    tok, single = first, []
+    for _ in range(6):
+        lg = gpt.decode(tok)
+        tok = int(np.argmax(lg))
+        single.append(tok)
+    assert [int(t) for t in ids] == single
+    assert np.array_equal(last, lg)
+    gpt.unloadBuffers()
+
+
 @pytest.mark.parametrize("name,n_layer", [("toy", 3), ("gpt2-117m", 2)])
 def test_persistent_decode_across_the_short_context_limit(device, name, n_layer):
     # the persistent kernel exists per context range (up to 512 positions, and beyond): steps on both sides of
