@@ -17,6 +17,7 @@ constexpr int PD_TOPK = 8;       // largest top_k the kernel samples from itself
 constexpr int PD_COLP = 256;     // floats of one workgroup's column parameters of a layer (4 phases x 32 columns x {bias, scale})
 constexpr int PD_KVBATCH = 4;    // key batches (of 32) a slice holds in registers: n_ctx <= 32*PD_KVBATCH*PD_SPLIT_LONG
 constexpr int PD_SHORT_KEYS = 32 * PD_KVBATCH * PD_SPLIT;  // longest context of the instantiation with PD_SPLIT slices
+constexpr int PD_NARROW_D = 1024;  // widest fp32 shape with LDS and registers to spare (table rows kept on the chip, host logits)
 constexpr int PD_TABLE_LDS_STEPS = 2;  // launches of at least this many steps keep part of the vocabulary table in LDS
 
 // How one linear layer is split over the workgroups: workgroup w finishes columns
@@ -78,6 +79,12 @@ struct PersistentArgs {
   const double* u;  // [nsteps], device memory (unused for top_k == 1)
   unsigned ebase;      // epoch of the last word published by earlier launches
   int pos0, nsteps;
+  // Results written straight into pinned host memory, so that a call of one step needs no copy behind the kernel
+  // (both may be null). host_logits[V]: the logits of the last step (shapes persistent_writes_host_logits names;
+  // needs rows_per_wg <= 4 d). host_done: workgroup 0 stores *err there once it has finished the last step, which
+  // it can only after every workgroup has published its last word; a launch that gave up leaves the word alone.
+  float* host_logits;
+  int* host_done;
 };
 
 PhaseGeom make_geom(int N, int K);
@@ -95,6 +102,8 @@ hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g,
 hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype, float* out, hipStream_t s);
 // Model shapes the persistent kernel is instantiated for.
 bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype);
+// Shapes whose kernel can write the last step's logits to host memory itself (PersistentArgs::host_logits).
+bool persistent_writes_host_logits(int d, int weight_dtype);
 // Epochs consumed by one decode step.
 inline unsigned persistent_epochs_per_step(int L) { return 5u * (unsigned)L + 1u; }
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s);

@@ -873,7 +873,7 @@ constexpr int table_rows_in_lds() {
   constexpr int spare = (160 * 1024 - 2048) / 4 - lds_floats<C>();
   // the wider shapes sit at the register limit, lose more to the extra code than the few rows that fit would give
   // them (d = 1280: 0.784 against 0.779 ms/token, int8 d = 1600: 1.00 against 0.80), and keep none
-  constexpr int rows = (spare > 0 && C::D <= 1024 && !C::I8) ? spare / C::D / NW * NW : 0;
+  constexpr int rows = (spare > 0 && C::D <= PD_NARROW_D && !C::I8) ? spare / C::D / NW * NW : 0;
   return rows > NW * PD_VOCAB_BATCH ? NW * PD_VOCAB_BATCH : rows;
 }
 
@@ -1404,6 +1404,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         tv[j] = -INFINITY;
         ti[j] = NOCAND;
       }
+      // the last step's logits also go to the caller's pinned memory, through LDS (narrow shapes only)
+      [[maybe_unused]] const bool to_host = LROWS > 0 && a.host_logits != nullptr && step == a.nsteps - 1;
       if constexpr (LROWS == 0) {
         // the shapes at the register limit keep this loop exactly as it was tuned: sharing the per-row code below
         // with them moved d = 1280 from 0.779 to 0.785 ms/token
@@ -1457,7 +1459,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         // one finished row: logit, running arg-max (rows come in ascending order per wave: the first index wins a
         // tie), top-k candidates
         auto tally = [&](float s, int row) {
-          if (lane == 0) a.logits[row] = s;
+          if (lane == 0) {
+            a.logits[row] = s;
+            if (to_host) xs1[row - v0] = s;  // (free since the last layer's second MLP product)
+          }
           if (s > best || besti == 0x7fffffff) {
             best = s;
             besti = row;
@@ -1551,6 +1556,12 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       }
       __syncthreads();
       ++ep;
+      if constexpr (LROWS > 0) {
+        // contiguous 256-byte stores per wave instead of 50257 single words crossing the bus; wave 0 stays out of it:
+        // it waits for its memory operations below, in front of the publish
+        if (to_host && wave > 0)
+          for (int r = tid - 64; r < v1 - v0; r += NT - 64) a.host_logits[v0 + r] = xs1[r];
+      }
       // Visibility of this token's cache rows to the next token. The slice that owned the new position appended k and v
       // of every layer with write-through device-scope stores issued by wave 0; wave 0 also publishes this workgroup's
       // word of the arg-max exchange below. Waiting here until every memory operation of the wave has completed
@@ -1703,6 +1714,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
     }
     __syncthreads();
   }
+  // Workgroup 0 is past the last exchange, so every workgroup has published its last word: the launch is complete
+  // unless a wait has expired somewhere meanwhile, which the error word says.
+  if (a.host_done && wg == 0 && tid == 0) *a.host_done = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // rowscale (may be null): the gamma of the LayerNorm in front of the matrix, folded in as
@@ -1845,6 +1859,8 @@ hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g,
   build_slab_i8_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(Wq, ldwq, K, g.N, g.cpw, g.S, total, slab);
   return hipGetLastError();
 }
+
+bool persistent_writes_host_logits(int d, int weight_dtype) { return weight_dtype == 0 && d <= PD_NARROW_D; }
 
 bool persistent_supports(int d, int n_head, int n_ctx, int weight_dtype) {
   if (n_ctx > 32 * PD_KVBATCH * PD_SPLIT_LONG) return false;

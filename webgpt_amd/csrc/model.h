@@ -59,6 +59,9 @@ struct Model {
   int32_t* pin = nullptr;
   float* logits_pin = nullptr;  // pinned host copy of the logits of the last call (V floats and the error word behind them)
   int32_t* ids_pin = nullptr;   // pinned host copy of the ids of a multi-step call (ctx ints)
+  // set by a persistent launch that writes its results to pinned memory itself, cleared by the read-back behind it:
+  // pin[1] holds the error word (or still -1: the kernel did not reach its end); logits_pin holds the logits
+  bool res_host_done = false, res_host_logits = false;
   unsigned epoch = 0;        // last epoch published by earlier launches
 
   // decode with one launch per block (decode_mode 0): the token's launches read the cache position from pos_dev and

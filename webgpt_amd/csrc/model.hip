@@ -432,8 +432,13 @@ static int setup_persistent(Model* m) {
 // Runs `steps` greedy decode steps from position m->pos with the persistent kernel.
 // The first token is in m->tok_dev[0]; chosen ids land in m->out_tok_dev.
 // top_k == 1: greedy. Otherwise u_dev holds the steps' uniform draws.
-static int decode_persistent(Model* m, int steps, int top_k = 1, double temperature = 1.0, const double* u_dev = nullptr, int token = -1) {
+// host_results: the call ends with a read-back (finish_timed, finish_steps): the kernel then reports its error word, and
+// where the shape allows the last step's logits, in pinned host memory itself instead of through copies behind it.
+static int decode_persistent(Model* m, int steps, int top_k = 1, double temperature = 1.0, const double* u_dev = nullptr, int token = -1,
+                             bool host_results = false) {
   PersistentArgs a = m->pa;
+  a.host_logits = nullptr;
+  a.host_done = nullptr;
   if (token >= 0) {  // the first token travels with the launch instead of through tok_dev
     a.tok = nullptr;
     a.tok_value = token;
@@ -465,7 +470,14 @@ static int decode_persistent(Model* m, int steps, int top_k = 1, double temperat
     if (a.u) a.u += short_steps;
     a.nsteps = steps - short_steps;
   }
+  if (host_results) {  // (the last launch of the call only)
+    m->pin[1] = -1;  // every earlier use of the word has completed: each call ends with a synchronisation
+    a.host_done = &m->pin[1];
+    if (persistent_writes_host_logits(m->d, m->p.weight_dtype) && a.rows_per_wg <= 4 * m->d) a.host_logits = m->logits_pin;
+  }
   LAUNCH(launch_decode_persistent(a, rt().stream));
+  m->res_host_done = a.host_done != nullptr;
+  m->res_host_logits = a.host_logits != nullptr;
   m->epoch += per_step * (unsigned)steps;
   return WGPT_OK;
 }
@@ -482,7 +494,7 @@ static int check_persistent(Model* m) {
     }
   }
 #endif
-  // the error word came back with the call's results (finish_timed)
+  // the error word came back with the call's results (read_back)
   const int herr = m->pin[1];
   if (herr != 0) {
     (void)hipMemset(m->perr, 0, sizeof(int));
@@ -490,43 +502,54 @@ static int check_persistent(Model* m) {
     m->decode_mode = 0;
     if (herr == -16)
       return fail(WGPT_ERR_DEVICE, "persistent decode kernel: its LDS rows are not 16-byte aligned (build problem); the persistent path is now disabled");
+    if (herr == -1)
+      return fail(WGPT_ERR_DEVICE, "persistent decode kernel: the launch did not run to its end; the persistent path is now disabled");
     return fail(WGPT_ERR_DEVICE, "persistent decode kernel: a bounded wait expired at epoch %d; the persistent path is now disabled", herr);
   }
   return WGPT_OK;
 }
 
-static int finish_timed(Model* m, float* logits) {
-  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
-  // the logits cross the bus into pinned memory (a copy into the caller's pageable buffer is staged by the
-  // runtime in pieces) and are handed over with a host copy
-  if (logits && m->perr) {  // the error word rides behind the logits
+// Brings the error word and, if asked for, the logits of the call to the host and drains the stream. The logits cross
+// the bus into pinned memory (a copy into the caller's pageable buffer is staged by the runtime in pieces) and are
+// handed over with a host copy; the error word rides behind them. What a persistent launch has written into pinned
+// memory itself (res_host_done, res_host_logits) is not copied again.
+static int read_back(Model* m, float* logits) {
+  const bool host_done = m->res_host_done, host_logits = m->res_host_logits;
+  m->res_host_done = m->res_host_logits = false;
+  const bool copy_logits = logits && !host_logits, copy_err = m->perr && !host_done;
+  if (copy_logits && copy_err) {
     WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * ((size_t)m->V + 1), hipMemcpyDeviceToHost, rt().stream));
   } else {
-    if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
-    if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
+    if (copy_logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
+    if (copy_err) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
   }
   WGPT_HIP(hipStreamSynchronize(rt().stream));
-  if (logits && m->perr) memcpy(&m->pin[1], m->logits_pin + m->V, sizeof(int));
+  if (copy_logits && copy_err) memcpy(&m->pin[1], m->logits_pin + m->V, sizeof(int));
+  if (host_done && m->pin[1] == -1) {
+    // the kernel did not reach its end: a wait has expired and the device's word says which
+    WGPT_HIP(hipMemcpy(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost));
+    if (m->pin[1] == 0) m->pin[1] = -1;
+  }
   if (logits) memcpy(logits, m->logits_pin, sizeof(float) * (size_t)m->V);
+  return WGPT_OK;
+}
+
+static int finish_timed(Model* m, float* logits) {
+  WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
+  const int rc = read_back(m, logits);
+  if (rc) return rc;
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   return WGPT_OK;
 }
 
-// The ids (and, if asked for, the logits) of a multi-step call come back through pinned memory: a copy into the caller's
-// pageable arrays is staged by the runtime and costs tens of microseconds per call. Ends with the stream drained.
+// The ids of a multi-step call come back through pinned memory as well: a copy into the caller's pageable array is
+// staged by the runtime and costs tens of microseconds per call. Ends with the stream drained.
 static int finish_steps(Model* m, int32_t* out_tokens, const int32_t* ids_dev, int steps, float* logits) {
   WGPT_HIP(hipEventRecord(m->ev1, rt().stream));
   WGPT_HIP(hipMemcpyAsync(m->ids_pin, ids_dev, sizeof(int32_t) * (size_t)steps, hipMemcpyDeviceToHost, rt().stream));
-  if (logits && m->perr) {  // the error word rides behind the logits
-    WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * ((size_t)m->V + 1), hipMemcpyDeviceToHost, rt().stream));
-  } else {
-    if (logits) WGPT_HIP(hipMemcpyAsync(m->logits_pin, m->logits, sizeof(float) * (size_t)m->V, hipMemcpyDeviceToHost, rt().stream));
-    if (m->perr) WGPT_HIP(hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream));
-  }
-  WGPT_HIP(hipStreamSynchronize(rt().stream));
+  const int rc = read_back(m, logits);
+  if (rc) return rc;
   memcpy(out_tokens, m->ids_pin, sizeof(int32_t) * (size_t)steps);
-  if (logits && m->perr) memcpy(&m->pin[1], m->logits_pin + m->V, sizeof(int));
-  if (logits) memcpy(logits, m->logits_pin, sizeof(float) * (size_t)m->V);
   WGPT_HIP(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
   return WGPT_OK;
 }
@@ -692,7 +715,7 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
     if ((rc = upload_position(m))) return rc;
   }
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
-  rc = m->decode_mode == 1 ? decode_persistent(m, 1, 1, 1.0, nullptr, token) : decode_token_blocks(m, m->pos);
+  rc = m->decode_mode == 1 ? decode_persistent(m, 1, 1, 1.0, nullptr, token, true) : decode_token_blocks(m, m->pos);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
@@ -719,7 +742,7 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   }
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   if (persistent) {
-    int rc = decode_persistent(m, steps, 1, 1.0, nullptr, token);
+    int rc = decode_persistent(m, steps, 1, 1.0, nullptr, token, true);
     if (rc) return rc;
   } else {
     for (int i = 0; i < steps; ++i) {
@@ -773,7 +796,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   const int pos_before = m->pos;
   int rc = WGPT_OK;
   if (in_kernel) {
-    rc = decode_persistent(m, steps, k, temperature, m->u_dev, token);
+    rc = decode_persistent(m, steps, k, temperature, m->u_dev, token, true);
   } else {
     for (int i = 0; i < steps && rc == WGPT_OK; ++i) {
       // one token per launch: the sampled id in tok_dev[0] is the next launch's input
