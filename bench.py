@@ -202,14 +202,16 @@ def main():
         "prefill_tflops": round(prefill_flops / (prefill_gpu_ms * 1e-3) / 1e12, 2),
         "prefill_frac_of_fp32_mfma_peak": round(prefill_flops / (prefill_gpu_ms * 1e-3) / MFMA_FP32_PEAK_FLOPS, 4),
         "host_loop_ms_per_token": {"mean": round(float(np.mean(per_tok)), 4), "p50": round(float(np.median(per_tok)), 4),
-                                   "note": "wgpt_decode per token incl. logits read-back over PCIe"} if per_tok else None,
+                                   "note": "wgpt_decode per token incl. the logits handed to the host over PCIe"} if per_tok else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_from": traffic_from,
                      "kernel": kernel_name,
                      "bytes_per_step": int(bytes_total / args.steps),
                      "note": "achieved = algorithmic bytes (weights + KV rows read) of the timed steps / HIP-event time of "
                              "the launch(es) that ran them; traffic = measured HBM bytes of one step (rocprofv3 FETCH_SIZE + "
-                             "WRITE_SIZE, profiles/), null where no counter run exists for the configuration"},
+                             "WRITE_SIZE, profiles/) as counted on single-step launches (a launch of several steps keeps "
+                             "up to a third of the vocabulary table in LDS and registers and reads that much less per step), "
+                             "null where no counter run exists for the configuration"},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt)
