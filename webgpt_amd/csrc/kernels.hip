@@ -2086,9 +2086,28 @@ void run_gemm(int M, int N, int K, const float* A, int lda, const void* W, int l
   }
   const bool big = (size_t)cdiv(M, 128) * cdiv(N, 128) >= 512;
   const int t = big ? 128 : 64;
+  constexpr int BKS = 32;  // K step of gemm_mfma
   int S = 1;
   const size_t tiles = (size_t)cdiv(M, t) * cdiv(N, t);
   while (workspace && S < 8 && tiles * S < 512 && K / (2 * S) >= 128) S *= 2;
+  if (workspace && M <= 448 && tiles <= 256) {
+    // Few rows: the workgroups of a launch all start together, one to a compute unit and a second one on some once
+    // there are more than 256 of them, and the launch lasts as long as the busiest unit. Any slice count that
+    // leaves whole K steps will do (three slices of c_attn at 128 rows are 216 workgroups of 8 steps, where four
+    // are 288 of 6, two of them on 32 units): the cheapest of rounds x (steps per slice + 4 for a round's prologue
+    // and epilogue). 117M T = 128: 0.895 -> 0.86 ms, T = 192: 1.07 -> 0.97; 1.5B T = 128: 6.67 -> 5.96; beyond
+    // ~450 rows several workgroups share a unit anyway and the doubling rule above measures better (T = 960:
+    // 2.56 against 2.63 ms).
+    long best = -1;
+    for (int c = 1; c <= 8; ++c) {
+      if (K % (BKS * c) != 0 || (c > 1 && K / c < 96)) continue;
+      const long cost = (long)cdiv(tiles * c, 256) * (K / (BKS * c) + 4);
+      if (best < 0 || cost < best) {
+        best = cost;
+        S = c;
+      }
+    }
+  }
   if (big) run_gemm_mfma<128, 128, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, kv, s);
   else run_gemm_mfma<64, 64, 32, I8W>(M, N, K, S, A, lda, W, ldw, wscale, bias, C, ldc, epi, resid, workspace, ln, kv, s);
 }
