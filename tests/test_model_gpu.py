@@ -255,19 +255,22 @@ def test_persistent_decode_across_the_short_context_limit(device, name, n_layer)
     cfg["n_layer"], cfg["n_ctx"] = n_layer, 1024
     gpt, _ = load(cfg, seed=9, random_ln=True)
     tokens = synth.tokens(12, "prompt", 540, cfg["vocab_size"])
-    out, ids, sampled = {}, {}, {}
+    out, ids, sampled, last = {}, {}, {}, {}
     u = np.random.default_rng(3).random(16)
     for mode in (0, 1):
         gpt.set_decode_mode(mode)
         gpt.prefill(tokens[:505])
         out[mode] = [gpt.decode(int(tokens[505 + i])) for i in range(14)]       # contexts 506..519
         lg = gpt.prefill(tokens[:500])
-        ids[mode] = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), 24)]   # one call, contexts 501..524
+        got, last[mode] = gpt.decode_greedy(int(np.argmax(lg)), 24, want_logits=True)   # one call, contexts 501..524
+        ids[mode] = [int(t) for t in got]
         gpt.prefill(tokens[:504])
         sampled[mode] = [int(t) for t in gpt.decode_sample(int(tokens[504]), len(u), 4, 0.9, u)]
     for i in range(14):
         assert close(out[1][i], out[0][i]), (i, worst(out[1][i], out[0][i]))
     assert ids[0] == ids[1]
+    # (the second of the call's two launches hands its logits to the host itself)
+    assert close(last[1], last[0]), worst(last[1], last[0])
     assert sampled[0] == sampled[1]
     gpt.unloadBuffers()
 
