@@ -1682,8 +1682,8 @@ __global__ __launch_bounds__(WG) void attention_decode_slice_kernel(int hs, int 
 
 // The final LayerNormBlock (model.js:224) and DeEmbedBlock (instructions.js:916-943) of a decode token in one
 // launch: every workgroup normalises the row itself while staging it (layernorm_kernel's order of operations), then
-// vocab_gemv_kernel's rows; the first workgroup finally advances the cache position (nothing later in the token
-// reads it).
+// vocab_gemv_kernel's rows; the first workgroup finally advances the cache position, if the caller passes one (nothing
+// later in the token reads it).
 __global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const float* __restrict__ x, const float* __restrict__ gamma,
                                                             const float* __restrict__ beta, const float* __restrict__ wte,
                                                             float* __restrict__ logits, int* pos) {
@@ -1761,7 +1761,7 @@ __global__ __launch_bounds__(WG) void vocab_gemv_ln_kernel(int V, int d, const f
     const float sum = wave_sum(acc[r]);
     if (lane == 0 && v0 + r < V) logits[v0 + r] = sum;
   }
-  if (blockIdx.x == 0 && threadIdx.x == 0) *pos += 1;
+  if (pos && blockIdx.x == 0 && threadIdx.x == 0) *pos += 1;
 }
 
 

@@ -192,8 +192,7 @@ static int forward_blocks(Model* m, int T, int pos0, bool want_taps) {
     LAUNCH(launch_vocab_gemv(m->V, d, m->ln + (size_t)(T - 1) * d, m->wte, m->logits, s));
   } else {
     // Only the last row is de-embedded (instructions.js:849-856).
-    LAUNCH(launch_layernorm(1, d, m->x + (size_t)(T - 1) * d, d, m->lnf_g, m->lnf_b, m->ln, d, s));
-    LAUNCH(launch_vocab_gemv(m->V, d, m->ln, m->wte, m->logits, s));
+    LAUNCH(launch_vocab_gemv_ln(m->V, d, m->x + (size_t)(T - 1) * d, m->lnf_g, m->lnf_b, m->wte, m->logits, nullptr, s));
   }
   return WGPT_OK;
 }
