@@ -61,6 +61,19 @@ def _dispatch_edge_shapes():
     return shapes
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 2304, 768), (64, 1536, 640), (128, 768, 672), (100, 768, 576), (448, 512, 768),
+                                   (449, 512, 768), (128, 1600, 6400), (33, 4800, 1600)])
+def test_fast_matmul_with_few_rows_and_odd_slice_counts(device, M, N, K):
+    # up to 448 rows the K range is cut into any number of slices that leaves whole steps of 32 (here 3, 5, 7, 6, ...),
+    # not only powers of two; 449 rows fall back to doubling. (Weights scaled with K: near a zero of the output the
+    # rounding of 6400 fp32 additions, in whatever order, is otherwise larger than the absolute tolerance.)
+    A, W, b = rnd(M, K), rnd(K, N, scale=0.05 * min(1.0, 1024.0 / K)), rnd(N)
+    inst = FastMatMulBlock.newInstance(M, N, K, init_tensor(A, [M, K]), init_tensor(W, [K, N]), init_tensor(b, [N]))
+    got = run(inst, (M, N))
+    want = ref.matmul_bias(A, W, b)
+    assert close(got, want), worst(got, want)
+
+
 @pytest.mark.parametrize("M,N,K", _dispatch_edge_shapes())
 def test_fast_matmul_around_kernel_choices(device, M, N, K):
     A, W, b = rnd(M, K), rnd(K, N, scale=0.05), rnd(N)
