@@ -388,8 +388,8 @@ static int setup_persistent(Model* m) {
     // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
     // curves are flat within a few percent around them and over context length);
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
-    static const int tuned[5][7] = {{16, 0, 20, 96, 20, 28, 48},    // d <= 768
-                                    {40, 0, 40, 96, 48, 40, 16},    // d = 1024
+    static const int tuned[5][7] = {{16, 4, 24, 96, 24, 24, 48},    // d <= 768
+                                    {32, 0, 40, 96, 40, 40, 4},     // d = 1024
                                     {20, 0, 40, 128, 24, 20, 40},   // d = 1280
                                     {16, 12, 20, 112, 20, 12, 4},   // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
