@@ -391,7 +391,7 @@ static int setup_persistent(Model* m) {
     static const int tuned[5][7] = {{16, 4, 24, 96, 24, 24, 48},    // d <= 768
                                     {32, 0, 40, 96, 40, 40, 4},     // d = 1024
                                     {20, 0, 40, 128, 24, 20, 40},   // d = 1280
-                                    {16, 12, 20, 112, 20, 12, 4},   // d = 1600, int8
+                                    {12, 12, 28, 96, 20, 12, 28},   // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
