@@ -53,6 +53,7 @@ def run_config(name, prompt_len, steps, oracle_at=(), max_prefill=0):
     for T in oracle_at:
         want = ref.forward(synth.model_params(cfg), oracle_weights(tensors, cfg), np.array(history[:T], np.int32))
         got = gpt.prefill(history[:T])
+        print(f"\nfull-size prefill parity {name} T={T}: worst |err| / (1e-5 + 1e-4 |want|) = {worst(got, want):.3f}", flush=True)
         assert close(got, want), (T, worst(got, want))
         assert greedy_ok(got, want)
     gpt.unloadBuffers()
@@ -67,15 +68,15 @@ def test_gpt2_117m_full():
 
 
 def test_gpt2_345m_full():
-    run_config("gpt2-345m", 512, 511, oracle_at=(16,))          # fills the context of 1024 exactly
+    run_config("gpt2-345m", 512, 511, oracle_at=(16, 512))          # fills the context of 1024 exactly
 
 
 def test_gpt2_774m_to_full_context():
-    run_config("gpt2-774m", 64, 959, oracle_at=(16,))           # decode up to the last position of the context
+    run_config("gpt2-774m", 64, 959, oracle_at=(16, 64))           # decode up to the last position of the context
 
 
 def test_gpt2_1p5b_int8_full():
-    run_config("gpt2-1.5b-int8", 128, 255, oracle_at=(16,))     # the configuration's 256 decode tokens
+    run_config("gpt2-1.5b-int8", 128, 255, oracle_at=(16, 128))     # the configuration's 256 decode tokens
 
 
 def test_gpt2_1p5b_fp32_across_512_positions():

@@ -253,7 +253,7 @@ def test_persistent_decode_across_the_short_context_limit(device, name, n_layer)
     # the limit, and multi-step launches that cross it, against the per-block path
     cfg = dict(synth.CONFIGS[name])
     cfg["n_layer"], cfg["n_ctx"] = n_layer, 1024
-    gpt, _ = load(cfg, seed=9, random_ln=True)
+    gpt, tensors = load(cfg, seed=9, random_ln=True)
     tokens = synth.tokens(12, "prompt", 540, cfg["vocab_size"])
     out, ids, sampled, last = {}, {}, {}, {}
     u = np.random.default_rng(3).random(16)
@@ -268,6 +268,14 @@ def test_persistent_decode_across_the_short_context_limit(device, name, n_layer)
         sampled[mode] = [int(t) for t in gpt.decode_sample(int(tokens[504]), len(u), 4, 0.9, u)]
     for i in range(14):
         assert close(out[1][i], out[0][i]), (i, worst(out[1][i], out[0][i]))
+    # both context ranges of the persistent kernel against the oracle itself: the full forward over the history
+    # (model.js:104-241) at a context below the limit of 512 positions and at one above it
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    for i in (0, 13):                                                            # contexts 506 and 519
+        want = ref.forward(p, w, tokens[:506 + i])
+        for mode in (1, 0):
+            assert close(out[mode][i], want), (name, mode, 506 + i, worst(out[mode][i], want))
+        assert greedy_ok(out[1][i], want)
     assert ids[0] == ids[1]
     # (the second of the call's two launches hands its logits to the host itself)
     assert close(last[1], last[0]), worst(last[1], last[0])

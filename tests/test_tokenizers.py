@@ -63,6 +63,28 @@ def test_js_tokenizers_agree_with_python():
     assert out["simple"] == {"ids": [4, 5, 7], "text": "hee", "n": 8}
 
 
+FULL_BPE = "/root/reference/weights/tokenization/vocab.bpe"
+# GPT-2's published encodings (the ids every GPT-2 tokenizer gives for these strings); they need merges far beyond
+# the first 1000, so they run only where the reference's complete merges file is readable
+PUBLISHED = {"Hello world": [15496, 995], " Hello": [18435],
+             "The quick brown fox jumps over the lazy dog.": [464, 2068, 7586, 21831, 18045, 625, 262, 16931, 3290, 13]}
+
+
+@pytest.mark.skipif(not os.access(FULL_BPE, os.R_OK), reason="the reference's complete vocab.bpe is not on this machine")
+def test_gpt2_published_ids_with_the_complete_merges_file():
+    t = GPT2Tokenizer().load(FULL_BPE)
+    assert t.getVocabSize() == 50257 and t.encoder["<|endoftext|>"] == 50256
+    for text, ids in PUBLISHED.items():
+        assert t.encode(text) == ids and t.decode(ids) == text, text
+    if NODE is not None:
+        r = subprocess.run([NODE, os.path.join(ROOT, "tests", "js", "tokenizer_checks.js"), FULL_BPE, *PUBLISHED],
+                           capture_output=True, text=True, timeout=120, cwd=ROOT)
+        assert r.returncode == 0, r.stderr[-2000:]
+        out = json.loads(r.stdout.strip().splitlines()[-1])
+        assert out["vocab_size"] == 50257 and out["eot"] == 50256
+        assert out["ids"] == list(PUBLISHED.values()) and out["round"] == list(PUBLISHED)
+
+
 @pytest.mark.gpu
 def test_generate_from_text(device):
     """generate(prompt: string) end to end (model.js:53-102) with the character tokenizer."""
