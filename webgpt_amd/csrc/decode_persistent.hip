@@ -45,6 +45,20 @@ __device__ __forceinline__ u64 ld_word(const u64* p) { return __hip_atomic_load(
 __device__ __forceinline__ void st_word(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void publish(u64* p, float v, unsigned epoch) { st_word(p, ((u64)epoch << 32) | __float_as_uint(v)); }
 
+// Three values and one epoch in 16 bytes, written by one 128-bit store of one lane and polled by one 128-bit load
+// (poll_triples): a naturally aligned 16-byte access of a lane is one transaction on both sides, so the epoch
+// validates the three values it travels with. What a hop costs beyond its latency goes with the number of poll
+// instructions, and a consumer reads a third fewer of these than of {value, epoch} pairs.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void publish3(u64* p, float v0, float v1, float v2, unsigned epoch) {
+  u32x4 pk;
+  pk.x = __float_as_uint(v0);
+  pk.y = __float_as_uint(v1);
+  pk.z = __float_as_uint(v2);
+  pk.w = epoch;
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(pk) : "memory");
+}
+
 // Streaming (non-temporal) 128-bit load: weights are read once per token and must
 // not displace the small hot data (parameters, instructions) from the caches.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -102,6 +116,22 @@ __device__ __forceinline__ void wave_sum_n(float (&v)[N]) {
   for (int i = 0; i < N; ++i) v[i] = dpp_add<0x143, 0xc>(v[i]);
 #pragma unroll
   for (int i = 0; i < N; ++i) v[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[i]), 63));
+}
+// Maximum / sum over each group of 8 adjacent lanes, every lane of the group gets it: lane ^ 1 and lane ^ 2 inside
+// the quad, then the mirrored lane of the half row, which lies in the group's other quad.
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float group8_max(float v) {
+  v = fmaxf(v, dpp_get<0xB1>(v));
+  v = fmaxf(v, dpp_get<0x4E>(v));
+  return fmaxf(v, dpp_get<0x141>(v));
+}
+__device__ __forceinline__ float group8_sum(float v) {
+  v += dpp_get<0xB1>(v);
+  v += dpp_get<0x4E>(v);
+  return v + dpp_get<0x141>(v);
 }
 // Sum over each row of 16 lanes, every lane of the row gets it (row rotations).
 __device__ __forceinline__ float row16_sum(float v) {
@@ -178,7 +208,8 @@ struct Shape {
   static_assert(H * SPLIT <= PD_GRID, "a workgroup per head and slice");
   static constexpr int SD = (D + SEG - 1) / SEG;      // segments of a D-long contraction
   static constexpr int SH = (HID + SEG - 1) / SEG;    // segments of a HID-long contraction
-  static constexpr int ATTW = H * SPLIT * (HS + 2);   // words of the attention exchange buffer
+  static constexpr int ATTW = H * SPLIT * (HS + 2);   // values of the attention exchange (three to a word)
+  static_assert((HS + 2) % 3 == 0, "a slice's values fill whole words of three");
   static_assert(HS == 64, "the attention phase is laid out for head size 64");
 };
 
@@ -221,7 +252,6 @@ __device__ __forceinline__ void static_for(F&& f) {
 // statement: the compiler does not track loads made in inline assembly, so none of the destinations may be touched
 // before the wait that ends the statement. (vmcnt(0) also covers the weight requests in flight: they were issued
 // earlier and return first anyway.)
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 template <int NL>
 struct WideLoads;
 #define WGPT_WL "global_load_dwordx4 "
@@ -318,6 +348,64 @@ __device__ __forceinline__ void poll_words(const u64* __restrict__ buf, unsigned
       for (int i = 0; i < n; ++i)
         if ((pending & (1u << (c0 + i))) && pk[i].y == epoch && pk[i].w == epoch) {
           *reinterpret_cast<float2*>(dst + 2 * (t + (c0 + i) * NT)) = make_float2(__uint_as_float(pk[i].x), __uint_as_float(pk[i].z));
+          pending &= ~(1u << (c0 + i));
+        }
+    });
+    if (pending) {
+      ++spins;
+      if (spins > spin_limit || bail_flag() ||
+          ((spins & 255u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+        sh.bail = 1;
+        atomicCAS(err, 0, (int)epoch);
+        break;
+      }
+    }
+  }
+}
+
+// The same for NQ words of three values (publish3). CPW = 0: word q carries values 3q .. 3q + 2 of dst. Otherwise
+// every producer owns CPW consecutive values of dst and publishes them as ceil(CPW / 3) words, the last one padded.
+template <int NQ, int CPW>
+__device__ __forceinline__ void poll_triples(const u64* __restrict__ buf, unsigned epoch, float* dst, int* err, int delay,
+                                             unsigned spin_limit) {
+  constexpr int NP = (NQ + NT - 1) / NT;
+  constexpr int CH = 7;
+  constexpr int T = (CPW + 2) / 3;
+  const int t = opaque(threadIdx.x);
+  unsigned pending = 0;
+  const u64* src[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const bool mine = i * NT + NT <= NQ || t + i * NT < NQ;
+    if (mine) pending |= 1u << i;
+    src[i] = buf + 2 * (mine ? t + i * NT : NQ - 1);
+  }
+  unsigned spins = 0;
+  nap(delay);
+  while (pending) {
+    static_for<(NP + CH - 1) / CH>([&](auto CI) {
+      constexpr int c0 = decltype(CI)::value * CH, n = NP - c0 < CH ? NP - c0 : CH;
+      u32x4 pk[n];
+      const u64* ps[n];
+#pragma unroll
+      for (int i = 0; i < n; ++i) ps[i] = src[c0 + i];
+      WideLoads<n>::run(pk, ps);
+#pragma unroll
+      for (int i = 0; i < n; ++i)
+        if ((pending & (1u << (c0 + i))) && pk[i].w == epoch) {
+          const int q = t + (c0 + i) * NT;
+          if constexpr (CPW % 3 == 0) {
+            float* d = dst + 3 * q;
+            d[0] = __uint_as_float(pk[i].x);
+            d[1] = __uint_as_float(pk[i].y);
+            d[2] = __uint_as_float(pk[i].z);
+          } else {
+            const int pw = q / T, r = q - pw * T;
+            float* d = dst + pw * CPW + 3 * r;
+            d[0] = __uint_as_float(pk[i].x);
+            if (3 * r + 1 < CPW) d[1] = __uint_as_float(pk[i].y);
+            if (3 * r + 2 < CPW) d[2] = __uint_as_float(pk[i].z);
+          }
           pending &= ~(1u << (c0 + i));
         }
     });
@@ -1182,28 +1270,31 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
         }
         __syncthreads();
-        if (tid < HS + 2) {
-          float M = -INFINITY;
+        if (wave == 0) {
+          // Wave 0 combines the eight: lane l takes element l of the output, lanes of equal l & 7 the factor
+          // exp(m_w - M) of wave w = l & 7 (one exponential per lane instead of eight in a row per element).
+          static_assert(HS == 64 && NW == 8, "one lane per element, eight waves");
+          const int lw = lane & (NW - 1);
+          const float mv = part[lw * (HS + 4) + HS];
+          const float M = group8_max(mv);
+          const float f = mv > -INFINITY ? fast_exp(mv - M) : 0.f;
+          const float lsum = group8_sum(part[lw * (HS + 4) + HS + 1] * f);
+          float o = 0.f;
 #pragma unroll
-          for (int w2 = 0; w2 < NW; ++w2) M = fmaxf(M, part[w2 * (HS + 4) + HS]);
-          float v = M;
-          if (tid != HS) {
-            const int c = tid < HS ? tid : HS + 1;
-            v = 0.f;
-#pragma unroll
-            for (int w2 = 0; w2 < NW; ++w2) {
-              const float mv = part[w2 * (HS + 4) + HS];
-              v += part[w2 * (HS + 4) + c] * (mv > -INFINITY ? fast_exp(mv - M) : 0.f);
-            }
-          }
-          publish(a.bufATT + (size_t)wg * (HS + 2) + tid, v, ep);
+          for (int w2 = 0; w2 < NW; ++w2)
+            o += part[w2 * (HS + 4) + lane] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), w2));
+          // (o[0..63], M, l) as 22 words of three values: word r = values 3r .. 3r + 2
+          const float a0 = __shfl(o, 3 * lane), a1 = __shfl(o, 3 * lane + 1), a2 = __shfl(o, 3 * lane + 2);
+          const bool lastw = lane == (HS + 2) / 3 - 1;
+          if (lane < (HS + 2) / 3)
+            publish3(a.bufATT + 2 * ((size_t)wg * ((HS + 2) / 3) + lane), a0, lastw ? M : a1, lastw ? lsum : a2, ep);
         }
       }
 
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
         [[maybe_unused]] constexpr int PH = PH_PROJ;
-        poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
+        poll_triples<C::ATTW / 3, 0>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -1318,7 +1409,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
         ++ep;
-        if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
+        {
+          constexpr int T = (PD::CPW + 2) / 3;  // words of three values per workgroup, the last one padded
+          static_assert(!PD::RAGGED, "every workgroup finishes CPW hidden units");
+          if (tid < T) {
+            const int c = 3 * opaque(tid);
+            publish3(a.bufH + 2 * (wg * T + tid), pubD[c], c + 1 < PD::CPW ? pubD[c + 1] : 0.f, c + 2 < PD::CPW ? pubD[c + 2] : 0.f, ep);
+          }
+        }
         TRACE5(4);
         if (!DUAL) nextE.all();
         else if (!SPREAD) nextE.late();
@@ -1343,7 +1441,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         };
         // (the last layer of the last step requests the first layer's share too and leaves it unused)
         const LoadA nextA(wX, li + 1 < a.L ? slab + a.slab_stride : slabs, ncA, wg, wave, lane);
-        poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
+        poll_triples<PD_GRID * ((PD::CPW + 2) / 3), PD::CPW>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
