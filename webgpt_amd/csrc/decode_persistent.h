@@ -32,7 +32,7 @@ struct PhaseGeom {
 //  int8 scales of the four matrices 3d, d, 4d, d].
 struct LayerParamOffsets {
   int bA, bC, bD, bE, ln1g, ln1b, ln2g, ln2b;
-  int sA, sC, sD, sE;  // per-column scales of the int8 variant (unused for fp32 weights)
+  int sA, sC, sD, sE;  // per-column scales of the int8 variant; for fp32 weights sA and sD hold the column sums of diag(gamma) W
   int stride;
 };
 __host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
@@ -92,8 +92,9 @@ size_t slab_float4s(const PhaseGeom& g);
 // Re-lays W[K, N] (row stride ldw) into the slab layout of geometry g; with rowscale
 // (the gamma of the LayerNorm in front of the matrix, or null) as diag(rowscale) W.
 hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const float* rowscale, float4* slab, hipStream_t s);
-// out[N] = bias + beta W: the beta of that LayerNorm folded into the bias.
-hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* beta, const float* bias, float* out, hipStream_t s);
+// out[N] = bias + beta W: the beta of that LayerNorm folded into the bias; colsum[N] = column sums of diag(gamma) W.
+hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* gamma, const float* beta, const float* bias, float* out,
+                        float* colsum, hipStream_t s);
 // Same for int8 words Wq[K, ldwq] (4 columns per word): one word per item lane.
 hipError_t build_slab_i8(const int32_t* Wq, int ldwq, int K, const PhaseGeom& g, int32_t* slab, hipStream_t s);
 // Biases and (int8) column scales / 127 of lparams re-laid per layer and workgroup: float t of a block is

@@ -435,6 +435,7 @@ struct WSet {
 // requested waits for every load in flight, the weights of the next phase included.)
 constexpr int LPW = PD_COLP / 8;  // columns of a phase per workgroup, at most
 
+constexpr bool LN_EPILOGUE = true;
 // Linear phases of a layer, in execution order.
 enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
 
@@ -443,13 +444,20 @@ enum { PH_QKV = 0, PH_PROJ = 1, PH_FC = 2, PH_FC2 = 3 };
 struct ColParams {
   float bias, scale;
 };
-template <bool I8>
+template <bool SECOND>
 __device__ __forceinline__ ColParams col_params(const float* colp, int ph, int c) {
   c &= LPW - 1;
   ColParams r;
   r.bias = colp[ph * LPW + c];
-  r.scale = I8 ? colp[(4 + ph) * LPW + c] : 1.f;
+  r.scale = SECOND ? colp[(4 + ph) * LPW + c] : 1.f;
   return r;
+}
+// A column behind a folded LayerNorm (fp32 slabs hold diag(gamma) W, the bias holds bias + beta W, and the second
+// slot the column sum S = sum_k gamma_k W_kc): with the row's mean and reciprocal standard deviation
+// sum_k ((x_k - mean) rstd) gamma_k W_kc = rstd (dot - mean S), so the statistics are reduced side by side with the
+// dot products instead of in two dependent reductions in front of them.
+__device__ __forceinline__ float finish_ln(float dot, float mean, float rstd, const ColParams& cp) {
+  return rstd * (dot - mean * cp.scale) + cp.bias;
 }
 // Finished value of a column from its dot product: the int8 column scale, the bias last.
 template <bool I8>
@@ -800,6 +808,44 @@ __device__ __forceinline__ float gemv_whole(const WS& ws, const float* xs, const
   return val;
 }
 
+// WHOLE phases behind a folded LayerNorm: the raw row against the wave's columns, and the row's sum and sum of
+// squares in the same reduction; lane cc returns the dot product of the wave's cc-th column, every lane the mean
+// and the reciprocal standard deviation (instructions.js:451-550: biased variance, eps inside the square root).
+template <class P, class WS>
+__device__ __forceinline__ float gemv_whole_ln(const WS& ws, const float* xs, int ncols, int wave, int lane, float& mean, float& rstd) {
+  static_assert(P::WHOLE, "phase is not laid out by whole columns");
+  const int l4 = opaque(lane) * 4;
+  float4 xr[P::S];
+#pragma unroll
+  for (int s2 = 0; s2 < P::S; ++s2) xr[s2] = *reinterpret_cast<const float4*>(xs + s2 * SEG + l4);  // (zero beyond K)
+  float red[2 + P::CW];
+  red[0] = 0.f;
+  red[1] = 0.f;
+#pragma unroll
+  for (int s2 = 0; s2 < P::S; ++s2) {
+    red[0] += (xr[s2].x + xr[s2].y) + (xr[s2].z + xr[s2].w);
+    red[1] += (xr[s2].x * xr[s2].x + xr[s2].y * xr[s2].y) + (xr[s2].z * xr[s2].z + xr[s2].w * xr[s2].w);
+  }
+  static_for<P::CW>([&](auto CC) {
+    constexpr int cc = decltype(CC)::value;
+    const bool valid = wave + cc * NW < (P::RAGGED ? ncols : P::CPW);
+    float acc = 0.f;
+    if (valid) static_for<P::S>([&](auto SG) {
+      constexpr int seg = decltype(SG)::value;
+      acc = item_sum<false>(acc, to_float4(ws.w[cc * P::S + seg]), xr[seg]);
+    });
+    red[2 + cc] = acc;
+  });
+  wave_sum_n(red);
+  mean = red[0] * (1.0f / (float)P::K);
+  const float var = fmaxf(__builtin_fmaf(-mean, mean, red[1] * (1.0f / (float)P::K)), 0.f);
+  rstd = fast_rsqrt(var + 1e-5f);
+  float val = 0.f;
+#pragma unroll
+  for (int cc = 0; cc < P::CW; ++cc) val = lane == cc ? red[2 + cc] : val;
+  return val;
+}
+
 // Other phases: per (column, wave) partial sums go to part[col * NW + wave]. The item
 // code exists once per wave with every index a constant: a phase is short, and what
 // it costs is instruction count (a runtime-indexed single copy measured 5-15 %
@@ -983,6 +1029,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS, SPREAD = PS::SPREAD;
   constexpr int SPN = 2, SPD = 3;  // share of a dealt-out request run that goes between the dot products
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
+  constexpr bool LNEPI = FOLD && LN_EPILOGUE;  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
   constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;  // floats of the staged exchange words
@@ -1145,12 +1192,13 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         const LoadC nextC(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         if (DUAL && !SPREAD) nextC.early();
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
-        const ColParams cp = col_params<I8>(colp, PH, fc);
-        float dot;
+        const ColParams cp = col_params<true>(colp, PH, fc);  // second slot: int8 scale, or the column sum of a folded LayerNorm
+        float dot, mean = 0.f, rstd = 1.f;
         if constexpr (SPREAD) dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part, nextC);
+        else if constexpr (LNEPI) dot = gemv_whole_ln<PA>(wX, xs0, ncA, wave, lane, mean, rstd);
         else dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part);
         TRACE5(2);
-        if (finA) pubA[fc] = finish<I8>(dot, cp);
+        if (finA) pubA[fc] = LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp);
         __syncthreads();
         ++ep;
         if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
@@ -1400,13 +1448,14 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE(1 + li * 8 + PH);
         const LoadE nextE(wY, slab + a.slab_offE, ncE, wg, wave, lane);
         if (DUAL && !SPREAD) nextE.early();
-        const ColParams cp = col_params<I8>(colp, PH, fc);
-        float dot;
+        const ColParams cp = col_params<true>(colp, PH, fc);
+        float dot, mean = 0.f, rstd = 1.f;
         const Leading<LoadE, SPN, SPD> leadE{nextE};
         if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, leadE);
+        else if constexpr (LNEPI) dot = gemv_whole_ln<PD>(wX, xs0, ncD, wave, lane, mean, rstd);
         else dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part);
         TRACE5(2);
-        if (finD) pubD[fc] = gelu_ref(finish<I8>(dot, cp));  // model.js:188
+        if (finD) pubD[fc] = gelu_ref(LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
         ++ep;
         {
@@ -1838,13 +1887,21 @@ __global__ void build_slab_kernel(const float* __restrict__ W, int ldw, int K, i
 
 // out[n] = bias[n] + sum_k beta[k] W[k][n]: the beta of the LayerNorm in front of the
 // matrix, folded into the bias (accumulated in double, rounded once).
-__global__ void fold_ln_bias_kernel(const float* __restrict__ W, int ldw, int K, int N, const float* __restrict__ beta,
-                                    const float* __restrict__ bias, float* __restrict__ out) {
+// colsum[n] = sum_k fl(gamma[k] W[k][n]): the sum of the column as the slab holds it (build_slab_kernel rounds the
+// same products), for the LayerNorm taken as an epilogue (finish_ln).
+__global__ void fold_ln_bias_kernel(const float* __restrict__ W, int ldw, int K, int N, const float* __restrict__ gamma,
+                                    const float* __restrict__ beta, const float* __restrict__ bias, float* __restrict__ out,
+                                    float* __restrict__ colsum) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= N) return;
-  double acc = 0.0;
-  for (int k = 0; k < K; ++k) acc += (double)beta[k] * (double)W[(size_t)k * ldw + n];
+  double acc = 0.0, sum = 0.0;
+  for (int k = 0; k < K; ++k) {
+    const float w = W[(size_t)k * ldw + n];
+    acc += (double)beta[k] * (double)w;
+    sum += (double)(w * gamma[k]);
+  }
   out[n] = (float)((double)bias[n] + acc);
+  colsum[n] = (float)sum;
 }
 
 // int8: item (w, j = c*S + seg, lane) is one word holding rows k..k+3 (k = seg*256 + lane*4)
@@ -1883,9 +1940,10 @@ __global__ void build_colparams_kernel(const float* __restrict__ lparams, int L,
                 : ph == PH_FC ? (kind ? po.sD : po.bD) : (kind ? po.sE : po.bE);
   const int col = wg * g.cpw + c;
   float v = 0.f;
-  if (c < g.cpw && col < g.N && (kind == 0 || i8)) {
+  // second slot: int8 column scales, or for fp32 the column sums of the two matrices behind a LayerNorm
+  if (c < g.cpw && col < g.N && (kind == 0 || i8 || ph == PH_QKV || ph == PH_FC)) {
     v = lparams[(size_t)layer * po.stride + off + col];
-    if (kind) v = v / 127.0f;  // other/int8-gemm.js:126-132 divides by 127 before the column scale is applied
+    if (kind && i8) v = v / 127.0f;  // other/int8-gemm.js:126-132 divides by 127 before the column scale is applied
   }
   out[idx] = v;
 }
@@ -1947,8 +2005,9 @@ hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const 
   return hipGetLastError();
 }
 
-hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* beta, const float* bias, float* out, hipStream_t s) {
-  fold_ln_bias_kernel<<<(unsigned)((N + 127) / 128), 128, 0, s>>>(W, ldw, K, N, beta, bias, out);
+hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* gamma, const float* beta, const float* bias, float* out,
+                        float* colsum, hipStream_t s) {
+  fold_ln_bias_kernel<<<(unsigned)((N + 127) / 128), 128, 0, s>>>(W, ldw, K, N, gamma, beta, bias, out, colsum);
   return hipGetLastError();
 }
 

@@ -346,8 +346,8 @@ static int setup_persistent(Model* m) {
     for (const auto& pt : parts)
       if (pt.src) WGPT_HIP(hipMemcpyAsync(lp + pt.off, pt.src, sizeof(float) * pt.n, hipMemcpyDeviceToDevice, rt().stream));
     if (!i8) {
-      LAUNCH(fold_ln_bias(l.attn.w, 3 * d, d, 3 * d, l.ln1_b, l.attn_b, lp + po.bA, rt().stream));
-      LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_b, l.fc_b, lp + po.bD, rt().stream));
+      LAUNCH(fold_ln_bias(l.attn.w, 3 * d, d, 3 * d, l.ln1_g, l.ln1_b, l.attn_b, lp + po.bA, lp + po.sA, rt().stream));
+      LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_g, l.ln2_b, l.fc_b, lp + po.bD, lp + po.sD, rt().stream));
     }
   }
   a.slabs = slabs;
