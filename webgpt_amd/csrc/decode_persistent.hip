@@ -1029,7 +1029,15 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   constexpr bool DUAL = PS::DUAL, I8 = C::I8, EKS = PS::EKS, SPREAD = PS::SPREAD;
   constexpr int SPN = 2, SPD = 3;  // share of a dealt-out request run that goes between the dot products
   constexpr bool FOLD = !I8;  // fp32 slabs carry the LayerNorm gamma, their biases the beta (see build_slab, fold_ln_bias)
-  constexpr bool LNEPI = FOLD && LN_EPILOGUE;  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln)
+  // hidden row and attention slices exchanged as words of three values (the fp32 d = 1600 shape, which lives on spilled
+  // registers, spills five times as much with them and keeps {value, epoch} pairs)
+  constexpr bool TRIPLE_H = I8 || D < 1600, TRIPLE_ATT = TRIPLE_H;
+  // Cached keys and values requested at the start of c_attn's phase instead of after its publish. Measured and off:
+  // the attention starts 0.2 us earlier (after the publish the rows, not q, set its start), but the requests of all
+  // 256 workgroups in front of the dot products cost more: 117M 0.1430 against 0.1396 ms/token, 345M 0.379 against 0.368,
+  // each with its poll delays re-tuned.
+  constexpr bool KV_EARLY = false;
+  constexpr bool LNEPI = FOLD && LN_EPILOGUE && D <= 1280;  // (the fp32 d = 1600 shape, short of registers, spills six times as much with it)  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
   constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;  // floats of the staged exchange words
@@ -1189,6 +1197,24 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         wait_loads();
         TRACE(1 + li * 8 + PH);
+        if constexpr (KV_EARLY) {
+          // This layer's cached keys and values of the slice, a whole phase before the attention needs them: they
+          // come from memory in 0.5-0.8 us, and requested after the publish they, not q, set the attention's start.
+          // No branch around the loads (the compiler would wait for them where its arms join): workgroups without
+          // the attention role, and lanes without a row, read one row of the positional table instead, finite values
+          // that a score of -inf multiplies by zero. (Ordinary loads: a cached row never changes once written and is
+          // only requested below the position, see the end-of-token exchange.)
+          const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
+#pragma unroll
+          for (int i = 0; i < MAXKV; ++i) {
+            const int j = c0 + g16 + 32 * i;
+            const bool row = att_role && i < nkv && j < c1 && j < pos;
+            const float* kp = row ? Kc + (size_t)j * HS + sub * 4 : a.wpe + sub * 4;
+            const float* vp = row ? Vc + (size_t)j * HS + sub * 4 : a.wpe + sub * 4;
+            kreg[i] = *reinterpret_cast<const float4*>(kp);
+            vreg[i] = *reinterpret_cast<const float4*>(vp);
+          }
+        }
         const LoadC nextC(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         if (DUAL && !SPREAD) nextC.early();
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
@@ -1206,7 +1232,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (!DUAL) nextC.all();
         else if (!SPREAD) nextC.late();
         TRACE5(5);
-        if (att_role) {
+        if (!KV_EARLY && att_role) {
           // this layer's cached keys and values of the slice
           const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
 #pragma unroll
@@ -1318,7 +1344,24 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
           }
         }
         __syncthreads();
-        if (wave == 0) {
+        if constexpr (!TRIPLE_ATT) {
+          if (tid < HS + 2) {
+            float M = -INFINITY;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) M = fmaxf(M, part[w2 * (HS + 4) + HS]);
+            float v = M;
+            if (tid != HS) {
+              const int c = tid < HS ? tid : HS + 1;
+              v = 0.f;
+#pragma unroll
+              for (int w2 = 0; w2 < NW; ++w2) {
+                const float mv = part[w2 * (HS + 4) + HS];
+                v += part[w2 * (HS + 4) + c] * (mv > -INFINITY ? fast_exp(mv - M) : 0.f);
+              }
+            }
+            publish(a.bufATT + (size_t)wg * (HS + 2) + tid, v, ep);
+          }
+        } else if (wave == 0) {
           // Wave 0 combines the eight: lane l takes element l of the output, lanes of equal l & 7 the factor
           // exp(m_w - M) of wave w = l & 7 (one exponential per lane instead of eight in a row per element).
           static_assert(HS == 64 && NW == 8, "one lane per element, eight waves");
@@ -1342,7 +1385,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
         [[maybe_unused]] constexpr int PH = PH_PROJ;
-        poll_triples<C::ATTW / 3, 0>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
+        if constexpr (TRIPLE_ATT) poll_triples<C::ATTW / 3, 0>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
+        else poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -1458,7 +1502,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (finD) pubD[fc] = gelu_ref(LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp));  // model.js:188
         __syncthreads();
         ++ep;
-        {
+        if constexpr (!TRIPLE_H) {
+          if (tid < ncD) publish(a.bufH + wg * PD::CPW + tid, pubD[tid], ep);
+        } else {
           constexpr int T = (PD::CPW + 2) / 3;  // words of three values per workgroup, the last one padded
           static_assert(!PD::RAGGED, "every workgroup finishes CPW hidden units");
           if (tid < T) {
@@ -1490,7 +1536,8 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         };
         // (the last layer of the last step requests the first layer's share too and leaves it unused)
         const LoadA nextA(wX, li + 1 < a.L ? slab + a.slab_stride : slabs, ncA, wg, wave, lane);
-        poll_triples<PD_GRID * ((PD::CPW + 2) / 3), PD::CPW>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
+        if constexpr (TRIPLE_H) poll_triples<PD_GRID * ((PD::CPW + 2) / 3), PD::CPW>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
+        else poll_words<HID>(a.bufH, ep, xs1, a.err, a.delay[5], a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -2035,6 +2082,9 @@ hipError_t build_colparams(const float* lparams, int L, int d, int weight_dtype,
 
 hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
   if (!persistent_supports(a.d, a.H, a.ctx, a.weight_dtype) || a.top_k < 1 || a.top_k > PD_TOPK) return hipErrorInvalidValue;
+#ifdef WGPT_ONLY_D  // experiments: one instantiation, a minute less per build
+  if (a.weight_dtype == 0 && a.d == WGPT_ONLY_D) return launch_t<WGPT_ONLY_D, WGPT_ONLY_D / 64, false>(a, s);
+#else
   if (a.weight_dtype == 1) return launch_t<1600, 25, true>(a, s);
   switch (a.d) {
     case 384: return launch_t<384, 6, false>(a, s);
@@ -2043,6 +2093,7 @@ hipError_t launch_decode_persistent(const PersistentArgs& a, hipStream_t s) {
     case 1280: return launch_t<1280, 20, false>(a, s);
     case 1600: return launch_t<1600, 25, false>(a, s);
   }
+#endif
   return hipErrorInvalidValue;
 }
 
