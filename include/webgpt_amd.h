@@ -92,6 +92,13 @@ int wgpt_residual(int M, int N, wgpt_buf a, wgpt_buf b, wgpt_buf out);
 int wgpt_layernorm(int M, int N, wgpt_buf x, wgpt_buf gamma, wgpt_buf beta, wgpt_buf out);
 /* SoftmaxBlock.newInstance(rows, cols, in) instructions.js:567-666. */
 int wgpt_softmax(int M, int N, wgpt_buf x, wgpt_buf out);
+/* SoftmaxBlock.newInstance(rows, cols, in, transpose = true): the same values stored transposed,
+ * out[i * M + row] (instructions.js:594), i.e. out is [N, M]. */
+int wgpt_softmax_t(int M, int N, wgpt_buf x, wgpt_buf out);
+/* transpose(array, rows, cols) of globals.js:80-94 on the device: out[c * rows + r] = in[r * cols + c].
+ * The reference transposes each vocabulary chunk on the host at load time (model.js:362-363); a host that
+ * is handed such [d, chunk] buffers turns them back into rows with this. */
+int wgpt_transpose(int rows, int cols, wgpt_buf in, wgpt_buf out);
 /* GeluBlock.newInstance(rows, cols, in) instructions.js:683-748. out may alias x. */
 int wgpt_gelu(int M, int N, wgpt_buf x, wgpt_buf out);
 /* EmbedBlock.newInstance(idx, T, d, ...) instructions.js:790-827: out[i] = wte[idx[i]] + wpe[i].
@@ -163,7 +170,9 @@ int wgpt_model_reset_cache(wgpt_model m);
 int wgpt_model_position(wgpt_model m, int* pos);
 /* Activation taps of the last wgpt_prefill (needs WGPT_FLAG_TAPS): names follow
  * other/validation/validation.js:183-205: tok_pos_emb, block<i>_{ln1,attn,r1,ln2,mlp,r2},
- * ln_f (each [T,d]); also kv<i>_k / kv<i>_v: the cache rows 0..pos-1 of layer i ([pos,d]). */
+ * ln_f (each [T,d]); also kv<i>_k / kv<i>_v: the cache rows 0..pos-1 of layer i ([pos,d]), and, without
+ * WGPT_FLAG_TAPS, `residual`: the residual stream after the last layer ([T,d]) of the last wgpt_prefill, which the
+ * reference copies into GPT.externalBuffer for its visualisation (model.js:211-222); valid until the next decode. */
 int wgpt_model_tap(wgpt_model m, const char* name, float* out, size_t n_floats);
 /* GPU time (HIP events on the library's stream) of the last prefill / decode /
  * decode_greedy call, in milliseconds, excluding the logits read-back. */

@@ -23,6 +23,33 @@ async function main() {
   // the reference's pass list, block by block, whole window recomputed
   const bw = gpt.loadBlockWeights(tensors);
   out.blocks24 = Array.from(await gpt.runBlocks(tokens, bw));
+  // the same pass list over the table held as the reference holds it: zero-padded [chunk, d] gather chunks and
+  // host-transposed [d, chunk] de-embedding chunks (model.js:298-364), here two chunks of 36 rows for 65
+  {
+    const { n_embd: d, vocab_size: V } = gpt.params;
+    const chunk = 36, padded = new Float32Array(2 * chunk * d);
+    padded.set(tensors["transformer.wte.weight"]);
+    const gather = [0, 1].map((i) => w.initTensor(padded.subarray(i * chunk * d, (i + 1) * chunk * d), [chunk, d]));
+    const transposed = [0, 1].map((i) => w.initTensor(Float32Array.from(w.transpose(padded.subarray(i * chunk * d, (i + 1) * chunk * d), chunk, d)), [d, chunk]));
+    out.chunked24 = Array.from(await gpt.runBlocks(tokens, bw, { vocab_chunk_size: chunk, embdBuffers: gather, deEmbeddingsBuffers: transposed }));
+    gather.concat(transposed).forEach((b) => b.destroy());
+    // softmax with the transposed store (instructions.js:594)
+    const sm = w.initTensor(new Float32Array([0, 1, 2, 3, 1, 1]), [2, 3]);
+    const inst = w.SoftmaxBlock.newInstance(2, 3, sm, true);
+    w.runPasses(inst.passes);
+    out.softmaxT = Array.from(inst.resultBuffer.download());
+    sm.destroy();
+    w.clearOperationCache();
+  }
+  // GPT.externalBuffer (model.js:211-222, visuals.js:48-50): run() leaves the last layer's residual rows there
+  {
+    const ext = new w.DeviceBuffer([cfg.n_ctx, cfg.n_embd]);
+    gpt.externalBuffer = ext;
+    out.extLogits = Array.from(await gpt.run(tokens.slice(0, 20)));
+    out.extRows = Array.from(ext.download(0, 4 * 20 * cfg.n_embd));
+    gpt.externalBuffer = undefined;
+    ext.destroy();
+  }
   // error path: the library's message becomes a thrown Error
   try { await gpt.run([cfg.vocab_size]); out.badToken = null; } catch (e) { out.badToken = e.message; }
   // generate() with top_k = 1, then the same continuation on the device

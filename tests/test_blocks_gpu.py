@@ -129,6 +129,53 @@ def test_softmax(device, M, N):
         assert np.count_nonzero(got[0, 2:]) == 0
 
 
+@pytest.mark.parametrize("M,N", [(1, 1), (3, 7), (24, 129), (65, 64)])
+def test_softmax_transposed_store(device, M, N):
+    # SoftmaxBlock.newInstance(rows, cols, in, transpose=true): out[i * M + row] (instructions.js:594)
+    x = rnd(M, N, scale=3.0)
+    inst = SoftmaxBlock.newInstance(M, N, init_tensor(x, [M, N]), True)
+    assert tuple(inst["resultBuffer"].dims) == (N, M)
+    got = run(inst, (N, M))
+    plain = run(SoftmaxBlock.newInstance(M, N, init_tensor(x, [M, N])), (M, N))
+    assert np.array_equal(got, plain.T)
+    want = ref.softmax(x).T
+    assert close(got, want, atol=1e-7), worst(got, want, atol=1e-7)
+
+
+def test_chunked_vocabulary_buffers_as_the_reference_builds_them(device):
+    """The reference holds the table as zero-padded chunks: [chunk, d] copies for the gather and host-transposed
+    [d, chunk] copies for the de-embedding (model.js:298-364; 50257 rows -> two chunks of 25132). Both blocks accept
+    such lists and give the single-table results bit for bit."""
+    V, d, T, ctx, chunk = 50257, 768, 9, 32, 25132
+    wte, wpe = rnd(V, d, scale=0.02), rnd(ctx, d, scale=0.02)
+    padded = np.zeros((2 * chunk, d), np.float32)
+    padded[:V] = wte
+    gather = [init_tensor(padded[i * chunk:(i + 1) * chunk], [chunk, d]) for i in range(2)]
+    transposed = [init_tensor(np.ascontiguousarray(padded[i * chunk:(i + 1) * chunk].T), [d, chunk]) for i in range(2)]
+    idx = np.array([0, V - 1, 17, 17, 25131, 25132, 40000, 3, 50256], np.int32)
+    wte_b, wpe_b = init_tensor(wte, [V, d]), init_tensor(wpe, [ctx, d])
+    inst = EmbedBlock.newInstance(idx, T, d, chunk, gather, wpe_b, ResidualBlock)
+    assert sum(p["flag"] == "copy" for p in inst["passes"]) == T + 1          # instructions.js:795-819
+    got = run(inst, (T, d))
+    assert np.array_equal(got, ref.embed(idx, wte, wpe))
+    assert np.array_equal(got, run(EmbedBlock.newInstance(idx, T, d, V, [wte_b], wpe_b, ResidualBlock), (T, d)))
+    x = rnd(T, d)
+    x_b = init_tensor(x, [T, d])
+    single = run(DeEmbedBlock.newInstance(d, V, V, T, V, x_b, [wte_b]), (V,))
+    for _ in range(2):   # the second instance finds the chunks' row form already made
+        inst = DeEmbedBlock.newInstance(d, V, 2 * chunk, T, chunk, x_b, transposed)
+        assert [p["flag"] for p in inst["passes"]] == ["compute", "copy"] * 2      # instructions.js:858-882
+        got = run(inst, (V,))
+        assert np.array_equal(got, single)
+    want = ref.deembed(x, wte)
+    assert close(got, want), worst(got, want)
+    with pytest.raises(ValueError, match="outside"):
+        EmbedBlock.newInstance(np.array([2 * chunk], np.int32), 1, d, chunk, gather, wpe_b, ResidualBlock)
+    for b in gather + transposed + [wte_b, wpe_b, x_b]:
+        b.destroy()
+    blocks.clearOperationCache()
+
+
 def test_embed_and_deembed(device):
     V, d, T, ctx = 50257, 768, 9, 32
     wte, wpe = rnd(V, d, scale=0.02), rnd(ctx, d, scale=0.02)

@@ -71,6 +71,15 @@ def test_js_gpt_on_gpu_matches_oracle():
     for key, want in (("logits16", want16), ("logits24", want24), ("blocks24", want24)):
         got = np.array(out[key], np.float32)
         assert close(got, want), (key, worst(got, want))
+    got = np.array(out["chunked24"], np.float32)
+    assert np.array_equal(got, np.array(out["blocks24"], np.float32))        # chunked table: same logits bit for bit
+    x = np.array([[0, 1, 2], [3, 1, 1]], np.float32)
+    assert np.allclose(np.array(out["softmaxT"]).reshape(3, 2), ref.softmax(x).T, rtol=1e-6, atol=1e-7)
+    want20, taps20, _ = ref.forward(p, w, tokens[:20], want_taps=True, want_kv=True)
+    rows = np.array(out["extRows"], np.float32).reshape(20, cfg["n_embd"])
+    want_rows = taps20[ref.tap_names(cfg["n_layer"]).index(f"block{cfg['n_layer'] - 1}_r2")]
+    assert close(rows, want_rows), worst(rows, want_rows)
+    assert close(np.array(out["extLogits"], np.float32), want20)
     assert "outside" in out["badToken"]
     assert out["generated"] == out["greedy"]
     hist = [int(t) for t in tokens[:8]]

@@ -283,6 +283,29 @@ def test_persistent_decode_across_the_short_context_limit(device, name, n_layer)
     gpt.unloadBuffers()
 
 
+def test_external_buffer_receives_the_last_residual_rows(device):
+    # model.js:211-222: with GPT.externalBuffer set (visuals.js:48-50) run() copies the residual stream after the
+    # last layer, [seq_length, n_embd], into it
+    from webgpt_amd.blocks import Buffer
+    cfg = dict(synth.CONFIGS["toy"])
+    cfg["n_layer"] = 2
+    gpt, tensors = load(cfg, seed=31)
+    w, p = oracle_weights(tensors, cfg), synth.model_params(cfg)
+    tokens = synth.tokens(8, "prompt", 21, cfg["vocab_size"])
+    plain = [gpt.run(tokens[:20]), gpt.run(tokens)]          # prefill, then a cached step
+    gpt.externalBuffer = Buffer([cfg["n_ctx"], cfg["n_embd"]])
+    for T in (20, 21):
+        want_logits, want_taps, _ = ref.forward(p, w, tokens[:T], want_taps=True, want_kv=True)
+        logits = gpt.run(tokens[:T])
+        rows = gpt.externalBuffer.download(count=T * cfg["n_embd"]).reshape(T, cfg["n_embd"])
+        want = want_taps[ref.tap_names(cfg["n_layer"]).index(f"block{cfg['n_layer'] - 1}_r2")]
+        assert close(rows, want), worst(rows, want)
+        assert close(logits, want_logits) and close(logits, plain[T - 20])
+    gpt.externalBuffer.destroy()
+    gpt.externalBuffer = None
+    gpt.unloadBuffers()
+
+
 def test_int8_persistent_decode_against_oracle(device):
     # width of the 1.5B int8 configuration, two layers: persistent int8 decode vs per-block int8 decode vs oracle
     cfg = dict(synth.CONFIGS["gpt2-1.5b-int8"])

@@ -52,6 +52,8 @@ _SIGNATURES = {
     "wgpt_residual": ([_int, _int, _u64, _u64, _u64], True),
     "wgpt_layernorm": ([_int, _int, _u64, _u64, _u64, _u64], True),
     "wgpt_softmax": ([_int, _int, _u64, _u64], True),
+    "wgpt_softmax_t": ([_int, _int, _u64, _u64], True),
+    "wgpt_transpose": ([_int, _int, _u64, _u64], True),
     "wgpt_gelu": ([_int, _int, _u64, _u64], True),
     "wgpt_embed": ([_ip, _int, _int, _int, _u64, _u64, _u64], True),
     "wgpt_deembed": ([_int, _int, _int, _u64, _u64, _u64], True),

@@ -32,6 +32,9 @@ class Buffer:
         if not self.destroyed:
             _lib.call("wgpt_free", self.handle)
             self.destroyed = True
+            if getattr(self, "rows", None) is not None:  # row form of a transposed vocabulary chunk (DeEmbedBlock)
+                self.rows.destroy()
+                self.rows = None
 
     def upload(self, data, offset=0):
         a = np.ascontiguousarray(data)
@@ -165,11 +168,11 @@ class SoftmaxBlockClass(Block):
         self.name = "softmax"
 
     def newInstance(self, rows, cols, inputBuffer, transpose=False):
-        if transpose:
-            raise NotImplementedError("transposed softmax output is not used by GPT.run() and is not provided")
-        resultBuffer = self.initResultBuffer([rows, cols])
+        # transpose: the same values stored as [cols, rows] (instructions.js:594)
+        resultBuffer = self.initResultBuffer([cols, rows] if transpose else [rows, cols])
         return {"resultBuffer": resultBuffer,
-                "passes": [_compute("wgpt_softmax", rows, cols, inputBuffer.handle, resultBuffer.handle)]}
+                "passes": [_compute("wgpt_softmax_t" if transpose else "wgpt_softmax", rows, cols, inputBuffer.handle,
+                                    resultBuffer.handle)]}
 
 
 class GeluBlockClass(Block):
@@ -191,17 +194,32 @@ class EmbedBlockClass(Block):
         self.name = "embed"
 
     def newInstance(self, idx, seq_length, n_embd, vocab_chunk_size, embdBuffers, posEmbdBuffer, ResidualBlock):
-        """instructions.js:790-827. `embdBuffers` is the list the reference passes; here it
-        holds the single un-chunked [V, d] table, and `vocab_chunk_size` is its row count."""
-        if len(embdBuffers) != 1:
-            raise ValueError("the embedding table is held as one buffer; pass [wte]")
+        """instructions.js:790-827. `embdBuffers` is either the single un-chunked [V, d] table (one fused
+        gather + add) or the reference's list of zero-padded [vocab_chunk_size, d] chunks (model.js:348-361):
+        then token i is row idx[i] % vocab_chunk_size of chunk floor(idx[i] / vocab_chunk_size), copied row by
+        row, and the positional rows are added by the ResidualBlock, as the reference does (795-821)."""
         ids = np.ascontiguousarray(idx, dtype=np.int32)
-        resultBuffer = self.initResultBuffer([seq_length, n_embd])
-        V = embdBuffers[0].dims[0]
-        return {"resultBuffer": resultBuffer,
-                "passes": [_compute("wgpt_embed", ids.ctypes.data_as(C.POINTER(C.c_int32)), seq_length, n_embd, V,
-                                    embdBuffers[0].handle, posEmbdBuffer.handle, resultBuffer.handle)],
-                "_keepalive": ids}
+        if len(embdBuffers) == 1:
+            resultBuffer = self.initResultBuffer([seq_length, n_embd])
+            V = embdBuffers[0].dims[0]
+            return {"resultBuffer": resultBuffer,
+                    "passes": [_compute("wgpt_embed", ids.ctypes.data_as(C.POINTER(C.c_int32)), seq_length, n_embd, V,
+                                        embdBuffers[0].handle, posEmbdBuffer.handle, resultBuffer.handle)],
+                    "_keepalive": ids}
+        row = 4 * n_embd
+        embdOutputBuffer = self.initBuffer(["storage", "copy_to"], [seq_length, n_embd])
+        posEmbdOutputBuffer = self.initBuffer(["storage", "copy_to"], [seq_length, n_embd])
+        passes = []
+        for i in range(seq_length):
+            chunk, within = divmod(int(ids[i]), vocab_chunk_size)
+            if int(ids[i]) < 0 or chunk >= len(embdBuffers):
+                raise ValueError("token id outside the embedding chunks")
+            passes.append({"flag": "copy", "src": embdBuffers[chunk], "srcOffset": row * within,
+                           "dst": embdOutputBuffer, "dstOffset": row * i, "size": row})
+        passes.append({"flag": "copy", "src": posEmbdBuffer, "srcOffset": 0, "dst": posEmbdOutputBuffer, "dstOffset": 0,
+                       "size": row * seq_length})
+        res = (ResidualBlock or globals()["ResidualBlock"]).newInstance(seq_length, n_embd, embdOutputBuffer, posEmbdOutputBuffer)
+        return {"resultBuffer": res["resultBuffer"], "passes": passes + res["passes"]}
 
 
 class DeEmbedBlockClass(Block):
@@ -210,14 +228,33 @@ class DeEmbedBlockClass(Block):
         self.name = "deembed"
 
     def newInstance(self, n_embd, vocab_size, padded_vocab_size, seq_length, vocab_chunk_size, embedBuffer, deEmbeddingsBuffers):
-        """instructions.js:844-888. `deEmbeddingsBuffers` holds the single [V, d] table
-        (no host-side transposes, no chunk copies)."""
-        if len(deEmbeddingsBuffers) != 1:
-            raise ValueError("the embedding table is held as one buffer; pass [wte]")
+        """instructions.js:844-888. `deEmbeddingsBuffers` is either the single [V, d] table (no host-side
+        transposes, no chunk copies) or the reference's list of transposed, zero-padded [d, vocab_chunk_size]
+        chunks (model.js:362-363). A chunk is turned back into rows on the device the first time it is seen
+        (wgpt_transpose; the row form is kept with the buffer, which the reference also makes once, at load), and
+        every chunk's logits go to their offset in the result, the last copy dropping the padding columns
+        (instructions.js:873-880). The products are the single-table kernel's, row by row: same logits bit for bit."""
         resultBuffer = self.initBuffer(["map_read", "copy_to"], [vocab_size])
-        return {"resultBuffer": resultBuffer,
-                "passes": [_compute("wgpt_deembed", n_embd, vocab_size, seq_length, embedBuffer.handle,
-                                    deEmbeddingsBuffers[0].handle, resultBuffer.handle)]}
+        if len(deEmbeddingsBuffers) == 1 and deEmbeddingsBuffers[0].dims[0] == vocab_size:
+            return {"resultBuffer": resultBuffer,
+                    "passes": [_compute("wgpt_deembed", n_embd, vocab_size, seq_length, embedBuffer.handle,
+                                        deEmbeddingsBuffers[0].handle, resultBuffer.handle)]}
+        passes = []
+        for i, chunkBuffer in enumerate(deEmbeddingsBuffers):
+            if tuple(chunkBuffer.dims) != (n_embd, vocab_chunk_size):
+                raise ValueError("a de-embedding chunk must be [n_embd, vocab_chunk_size]")
+            if getattr(chunkBuffer, "rows", None) is None:
+                chunkBuffer.rows = Buffer([vocab_chunk_size, n_embd])
+                _lib.call("wgpt_transpose", n_embd, vocab_chunk_size, chunkBuffer.handle, chunkBuffer.rows.handle)
+            valid = min(vocab_chunk_size, vocab_size - i * vocab_chunk_size)
+            if valid <= 0:
+                break
+            chunkResultBuffer = self.initResultBuffer([valid])
+            passes.append(_compute("wgpt_deembed", n_embd, valid, seq_length, embedBuffer.handle, chunkBuffer.rows.handle,
+                                   chunkResultBuffer.handle))
+            passes.append({"flag": "copy", "src": chunkResultBuffer, "srcOffset": 0, "dst": resultBuffer,
+                           "dstOffset": 4 * i * vocab_chunk_size, "size": 4 * valid})
+        return {"resultBuffer": resultBuffer, "passes": passes}
 
 
 class AttentionBlockClass(Block):

@@ -237,8 +237,34 @@ int wgpt_softmax(int M, int N, wgpt_buf x, wgpt_buf out) {
   float* po = F(out, n, "wgpt_softmax(out)");
   if (!px || !po) return WGPT_ERR_ARG;
   if (px == po) return fail(WGPT_ERR_ARG, "wgpt_softmax: out must not alias x");
-  hipError_t e = launch_softmax(M, N, px, po, rt().stream);
+  hipError_t e = launch_softmax(M, N, px, po, false, rt().stream);
   if (e != hipSuccess) return fail(WGPT_ERR_HIP, "softmax launch: %s", hipGetErrorString(e));
+  return WGPT_OK;
+}
+
+int wgpt_softmax_t(int M, int N, wgpt_buf x, wgpt_buf out) {
+  WGPT_REQUIRE_INIT();
+  if (M < 1 || N < 1) return fail(WGPT_ERR_ARG, "wgpt_softmax_t: M and N must be positive");
+  const size_t n = (size_t)M * N;
+  const float* px = F(x, n, "wgpt_softmax_t(x)");
+  float* po = F(out, n, "wgpt_softmax_t(out)");
+  if (!px || !po) return WGPT_ERR_ARG;
+  if (px == po) return fail(WGPT_ERR_ARG, "wgpt_softmax_t: out must not alias x");
+  hipError_t e = launch_softmax(M, N, px, po, true, rt().stream);
+  if (e != hipSuccess) return fail(WGPT_ERR_HIP, "softmax launch: %s", hipGetErrorString(e));
+  return WGPT_OK;
+}
+
+int wgpt_transpose(int rows, int cols, wgpt_buf in, wgpt_buf out) {
+  WGPT_REQUIRE_INIT();
+  if (rows < 1 || cols < 1) return fail(WGPT_ERR_ARG, "wgpt_transpose: rows and cols must be positive");
+  const size_t n = (size_t)rows * cols;
+  const float* pi = F(in, n, "wgpt_transpose(in)");
+  float* po = F(out, n, "wgpt_transpose(out)");
+  if (!pi || !po) return WGPT_ERR_ARG;
+  if (pi == po) return fail(WGPT_ERR_ARG, "wgpt_transpose: out must not alias in");
+  hipError_t e = launch_transpose(rows, cols, pi, po, rt().stream);
+  if (e != hipSuccess) return fail(WGPT_ERR_HIP, "transpose launch: %s", hipGetErrorString(e));
   return WGPT_OK;
 }
 

@@ -60,7 +60,8 @@ hipError_t launch_residual(size_t n4, const float* a, const float* b, float* out
 hipError_t launch_gelu(size_t n4, const float* x, float* out, hipStream_t s);
 hipError_t launch_layernorm(int M, int N, const float* x, int ldx, const float* gamma, const float* beta, float* out, int ldo,
                             hipStream_t s);
-hipError_t launch_softmax(int M, int N, const float* x, float* out, hipStream_t s);
+hipError_t launch_softmax(int M, int N, const float* x, float* out, bool transpose, hipStream_t s);
+hipError_t launch_transpose(int rows, int cols, const float* in, float* out, hipStream_t s);
 // out[i,:] = wte[idx[i],:] + wpe[pos0+i,:]; idx on the device.
 hipError_t launch_embed(const int32_t* idx, int T, int d, int pos0, const float* wte, const float* wpe, float* out, hipStream_t s);
 // logits[v] = x . wte[v,:]

@@ -860,7 +860,9 @@ __global__ __launch_bounds__(WG) void layernorm_kernel(int N, const float* __res
 
 // SoftmaxBlock, instructions.js:618-663: max from -3.402823e38, sum of exp(x - max),
 // out = exp(x - max) / sum with the exponential recomputed and a true division.
-__global__ __launch_bounds__(WG) void softmax_kernel(int N, const float* __restrict__ x, float* __restrict__ out) {
+// TRANSPOSE: the store of instructions.js:594 with `transpose` set: element i of row r goes to out[i * M + r].
+template <bool TRANSPOSE>
+__global__ __launch_bounds__(WG) void softmax_kernel(int M, int N, const float* __restrict__ x, float* __restrict__ out) {
   __shared__ float sh[NWAVE];
   const float* xr = x + (size_t)blockIdx.x * N;
   float* orow = out + (size_t)blockIdx.x * N;
@@ -870,7 +872,23 @@ __global__ __launch_bounds__(WG) void softmax_kernel(int N, const float* __restr
   float s = 0.f;
   for (int i = threadIdx.x; i < N; i += WG) s += expf(xr[i] - m);
   s = block_sum(s, sh);
-  for (int i = threadIdx.x; i < N; i += WG) orow[i] = expf(xr[i] - m) / s;
+  for (int i = threadIdx.x; i < N; i += WG) {
+    const float v = expf(xr[i] - m) / s;
+    if (TRANSPOSE) out[(size_t)i * M + blockIdx.x] = v;
+    else orow[i] = v;
+  }
+}
+
+// out[c * rows + r] = in[r * cols + c] through a 32 x 32 tile of LDS (the host-side transpose of globals.js:80-94).
+__global__ __launch_bounds__(256) void transpose_kernel(int rows, int cols, const float* __restrict__ in, float* __restrict__ out) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  for (int k = ty; k < 32; k += 8)
+    if (r0 + k < rows && c0 + tx < cols) tile[k][tx] = in[(size_t)(r0 + k) * cols + c0 + tx];
+  __syncthreads();
+  for (int k = ty; k < 32; k += 8)
+    if (c0 + k < cols && r0 + tx < rows) out[(size_t)(c0 + k) * rows + r0 + tx] = tile[tx][k];
 }
 
 // EmbedBlock, instructions.js:795-821: gather + positional add in one pass.
@@ -2150,8 +2168,14 @@ hipError_t launch_layernorm(int M, int N, const float* x, int ldx, const float* 
   return hipGetLastError();
 }
 
-hipError_t launch_softmax(int M, int N, const float* x, float* out, hipStream_t s) {
-  softmax_kernel<<<M, WG, 0, s>>>(N, x, out);
+hipError_t launch_transpose(int rows, int cols, const float* in, float* out, hipStream_t s) {
+  transpose_kernel<<<dim3((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32)), 256, 0, s>>>(rows, cols, in, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_softmax(int M, int N, const float* x, float* out, bool transpose, hipStream_t s) {
+  if (transpose) softmax_kernel<true><<<M, WG, 0, s>>>(M, N, x, out);
+  else softmax_kernel<false><<<M, WG, 0, s>>>(M, N, x, out);
   return hipGetLastError();
 }
 

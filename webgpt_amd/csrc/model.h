@@ -32,6 +32,7 @@ struct Model {
   int decode_mode = 0;
   int pos = 0;     // positions held by the KV cache
   int tap_T = 0;   // rows of the recorded taps (0 = none)
+  int x_rows = 0;  // rows of the residual stream the last prefill left in x (0 once a decode step has run)
 
   float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
   std::vector<LayerW> layers;

@@ -691,12 +691,14 @@ int wgpt_prefill(wgpt_model h, const int32_t* tokens, int T, float* logits) {
   WGPT_HIP(hipEventRecord(m->ev0, rt().stream));
   m->pos = 0;
   m->tap_T = 0;
+  m->x_rows = 0;
   int rc = forward_blocks(m, T, 0, true);
   if (rc) return rc;
   rc = finish_timed(m, logits);
   if (rc) return rc;
   m->pos = T;
   m->tap_T = m->taps ? T : 0;
+  m->x_rows = T;
   return WGPT_OK;
 }
 
@@ -704,6 +706,7 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode: token id %d outside [0, %d)", token, m->V);
   if (m->pos >= m->ctx) return fail(WGPT_ERR_STATE, "wgpt_decode: context of %d positions is full; prefill a slid window", m->ctx);
@@ -727,6 +730,7 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: token id %d outside [0, %d)", token, m->V);
   if (steps < 1 || !out_tokens) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: steps >= 1 and out_tokens required");
@@ -767,6 +771,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_sample: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: token id %d outside [0, %d)", token, m->V);
   if (steps < 1 || !out_tokens || !u) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: steps >= 1, u and out_tokens required");
@@ -827,6 +832,7 @@ int wgpt_model_reset_cache(wgpt_model h) {
   if (!m) return WGPT_ERR_ARG;
   m->pos = 0;
   m->tap_T = 0;
+  m->x_rows = 0;
   return WGPT_OK;
 }
 
@@ -860,6 +866,12 @@ int wgpt_model_tap(wgpt_model h, const char* name, float* out, size_t n_floats) 
                                 sizeof(float) * m->hs, sizeof(float) * m->hs, (size_t)m->pos, hipMemcpyDeviceToHost, rt().stream));
     WGPT_HIP(hipStreamSynchronize(rt().stream));
     return WGPT_OK;
+  } else if (n == "residual") {
+    // the residual stream after the last layer as the last prefill left it: what the reference copies into
+    // GPT.externalBuffer (model.js:211-222); needs no WGPT_FLAG_TAPS
+    if (m->x_rows == 0) return fail(WGPT_ERR_STATE, "wgpt_model_tap: 'residual' holds the rows of the last wgpt_prefill until the next decode step");
+    src = m->x;
+    count = (size_t)m->x_rows * d;
   } else {
     if (!m->taps || m->tap_T == 0) return fail(WGPT_ERR_STATE, "wgpt_model_tap: no taps recorded (WGPT_FLAG_TAPS and a prefill are needed)");
     const size_t T = m->tap_T;

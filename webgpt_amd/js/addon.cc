@@ -30,7 +30,7 @@ void* g_lib = nullptr;
   X(wgpt_model_reset_cache) X(wgpt_model_position) X(wgpt_model_tap) X(wgpt_model_last_gpu_ms)          \
   X(wgpt_model_decode_bytes) X(wgpt_model_set_decode_mode) X(wgpt_model_destroy) X(wgpt_synth_normal)   \
   X(wgpt_synth_tokens) X(wgpt_synth_int8_packed) X(wgpt_synth_uniform) X(wgpt_synth_tensor_id)   \
-  X(wgpt_decode_sample) X(wgpt_sample_topk) X(wgpt_matmul_bias_noalloc)
+  X(wgpt_decode_sample) X(wgpt_sample_topk) X(wgpt_matmul_bias_noalloc) X(wgpt_softmax_t) X(wgpt_transpose)
 
 #define DECL(name) decltype(&::name) p_##name = nullptr;
 WGPT_FUNCS(DECL)
@@ -179,6 +179,8 @@ FN(DequantI8) { Args a(env, info); int K = a.i32(0), N = a.i32(1); uint64_t q = 
 FN(Residual) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), y = a.u64(3), o = a.u64(4); if (!a.ok) return nullptr; if (failed(env, p_wgpt_residual(M, N, x, y, o))) return nullptr; return undefined(env); }
 FN(LayerNorm) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), g = a.u64(3), b = a.u64(4), o = a.u64(5); if (!a.ok) return nullptr; if (failed(env, p_wgpt_layernorm(M, N, x, g, b, o))) return nullptr; return undefined(env); }
 FN(Softmax) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), o = a.u64(3); if (!a.ok) return nullptr; if (failed(env, p_wgpt_softmax(M, N, x, o))) return nullptr; return undefined(env); }
+FN(SoftmaxT) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), o = a.u64(3); if (!a.ok) return nullptr; if (failed(env, p_wgpt_softmax_t(M, N, x, o))) return nullptr; return undefined(env); }
+FN(Transpose) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), o = a.u64(3); if (!a.ok) return nullptr; if (failed(env, p_wgpt_transpose(M, N, x, o))) return nullptr; return undefined(env); }
 FN(Gelu) { Args a(env, info); int M = a.i32(0), N = a.i32(1); uint64_t x = a.u64(2), o = a.u64(3); if (!a.ok) return nullptr; if (failed(env, p_wgpt_gelu(M, N, x, o))) return nullptr; return undefined(env); }
 FN(Embed) {  // (Int32Array idx, T, d, V, wte, wpe, out)
   Args a(env, info);
@@ -391,7 +393,7 @@ napi_value InitModule(napi_env env, napi_value exports) {
       {"load", Load}, {"exports", Exports}, {"init", Init}, {"shutdown", Shutdown}, {"sync", Sync}, {"deviceInfo", DeviceInfo},
       {"alloc", Alloc}, {"free", Free}, {"upload", Upload}, {"download", Download}, {"copy", Copy},
       {"wgpt_matmul_bias", MatmulBias}, {"wgpt_matmul_bias_noalloc", MatmulBiasNoAlloc}, {"wgpt_matmul_bias_i8", MatmulBiasI8}, {"wgpt_dequant_i8", DequantI8},
-      {"wgpt_residual", Residual}, {"wgpt_layernorm", LayerNorm}, {"wgpt_softmax", Softmax}, {"wgpt_gelu", Gelu},
+      {"wgpt_residual", Residual}, {"wgpt_layernorm", LayerNorm}, {"wgpt_softmax", Softmax}, {"wgpt_softmax_t", SoftmaxT}, {"wgpt_transpose", Transpose}, {"wgpt_gelu", Gelu},
       {"wgpt_embed", Embed}, {"wgpt_deembed", DeEmbed}, {"wgpt_attention", Attention},
       {"modelCreate", ModelCreate}, {"modelSetTensor", ModelSetTensor}, {"modelFinalize", ModelFinalize},
       {"modelDestroy", ModelDestroy}, {"modelResetCache", ModelResetCache}, {"modelSetDecodeMode", ModelSetDecodeMode},

@@ -18,6 +18,10 @@ class DeviceBuffer {
   destroy() {
     if (!this.destroyed) native.free(this.handle);
     this.destroyed = true;
+    if (this.rows) {  // row form of a transposed vocabulary chunk (DeEmbedBlock)
+      this.rows.destroy();
+      this.rows = null;
+    }
   }
   upload(typedArray, offset = 0) {
     native.upload(this.handle, offset, typedArray);
@@ -147,10 +151,10 @@ class SoftmaxBlockClass extends Block {
     super();
     this.name = "softmax";
   }
+  // transpose: the same values stored as [cols, rows] (instructions.js:594)
   newInstance(rows, cols, inputBuffer, transpose = false) {
-    if (transpose) throw new Error("transposed softmax output is not used by GPT.run() and is not provided");
-    const resultBuffer = this.initResultBuffer([rows, cols]);
-    return { resultBuffer, passes: [compute("wgpt_softmax", rows, cols, inputBuffer.handle, resultBuffer.handle)] };
+    const resultBuffer = this.initResultBuffer(transpose ? [cols, rows] : [rows, cols]);
+    return { resultBuffer, passes: [compute(transpose ? "wgpt_softmax_t" : "wgpt_softmax", rows, cols, inputBuffer.handle, resultBuffer.handle)] };
   }
 }
 
@@ -171,15 +175,31 @@ class EmbedBlockClass extends Block {
     super();
     this.name = "embed";
   }
-  // embdBuffers holds the single un-chunked [V, d] table; vocab_chunk_size is its row count.
+  // embdBuffers is either the single un-chunked [V, d] table (one fused gather + add) or the reference's list of
+  // zero-padded [vocab_chunk_size, d] chunks (model.js:348-361): then token i is row idx[i] % vocab_chunk_size of chunk
+  // floor(idx[i] / vocab_chunk_size), copied row by row, and the positional rows are added by the ResidualBlock, as
+  // the reference does (instructions.js:795-821).
   newInstance(idx, seq_length, n_embd, vocab_chunk_size, embdBuffers, posEmbdBuffer, ResidualBlock) {
-    if (embdBuffers.length !== 1) throw new Error("the embedding table is held as one buffer; pass [wte]");
-    const ids = Int32Array.from(idx);
-    const resultBuffer = this.initResultBuffer([seq_length, n_embd]);
-    return {
-      resultBuffer,
-      passes: [compute("wgpt_embed", ids, seq_length, n_embd, embdBuffers[0].dims[0], embdBuffers[0].handle, posEmbdBuffer.handle, resultBuffer.handle)],
-    };
+    if (embdBuffers.length === 1) {
+      const ids = Int32Array.from(idx);
+      const resultBuffer = this.initResultBuffer([seq_length, n_embd]);
+      return {
+        resultBuffer,
+        passes: [compute("wgpt_embed", ids, seq_length, n_embd, embdBuffers[0].dims[0], embdBuffers[0].handle, posEmbdBuffer.handle, resultBuffer.handle)],
+      };
+    }
+    const row = 4 * n_embd;
+    const embdOutputBuffer = this.initBuffer(["storage", "copy_to"], [seq_length, n_embd]);
+    const posEmbdOutputBuffer = this.initBuffer(["storage", "copy_to"], [seq_length, n_embd]);
+    const passes = [];
+    for (let i = 0; i < seq_length; i++) {
+      const chunk = Math.floor(idx[i] / vocab_chunk_size);
+      if (!(idx[i] >= 0) || chunk >= embdBuffers.length) throw new Error("token id outside the embedding chunks");
+      passes.push({ flag: "copy", src: embdBuffers[chunk], srcOffset: row * (idx[i] % vocab_chunk_size), dst: embdOutputBuffer, dstOffset: row * i, size: row });
+    }
+    passes.push({ flag: "copy", src: posEmbdBuffer, srcOffset: 0, dst: posEmbdOutputBuffer, dstOffset: 0, size: row * seq_length });
+    const res = ResidualBlock.newInstance(seq_length, n_embd, embdOutputBuffer, posEmbdOutputBuffer);
+    return { resultBuffer: res.resultBuffer, passes: passes.concat(res.passes) };
   }
 }
 
@@ -188,11 +208,31 @@ class DeEmbedBlockClass extends Block {
     super();
     this.name = "deembed";
   }
-  // deEmbeddingsBuffers holds the single [V, d] table (no host transposes, no chunk copies).
+  // deEmbeddingsBuffers is either the single [V, d] table (no host transposes, no chunk copies) or the reference's
+  // list of transposed, zero-padded [d, vocab_chunk_size] chunks (model.js:362-363). A chunk is turned back into rows
+  // on the device the first time it is seen (wgpt_transpose; the row form is kept with the buffer, which the
+  // reference also makes once, at load), and every chunk's logits go to their offset in the result, the last copy
+  // dropping the padding columns (instructions.js:873-880). Same kernel row by row: same logits bit for bit.
   newInstance(n_embd, vocab_size, padded_vocab_size, seq_length, vocab_chunk_size, embedBuffer, deEmbeddingsBuffers) {
-    if (deEmbeddingsBuffers.length !== 1) throw new Error("the embedding table is held as one buffer; pass [wte]");
     const resultBuffer = this.initBuffer(["map_read", "copy_to"], [vocab_size]);
-    return { resultBuffer, passes: [compute("wgpt_deembed", n_embd, vocab_size, seq_length, embedBuffer.handle, deEmbeddingsBuffers[0].handle, resultBuffer.handle)] };
+    if (deEmbeddingsBuffers.length === 1 && deEmbeddingsBuffers[0].dims[0] === vocab_size) {
+      return { resultBuffer, passes: [compute("wgpt_deembed", n_embd, vocab_size, seq_length, embedBuffer.handle, deEmbeddingsBuffers[0].handle, resultBuffer.handle)] };
+    }
+    const passes = [];
+    for (let i = 0; i < deEmbeddingsBuffers.length; i++) {
+      const chunkBuffer = deEmbeddingsBuffers[i];
+      if (chunkBuffer.dims[0] !== n_embd || chunkBuffer.dims[1] !== vocab_chunk_size) throw new Error("a de-embedding chunk must be [n_embd, vocab_chunk_size]");
+      if (!chunkBuffer.rows) {
+        chunkBuffer.rows = new DeviceBuffer([vocab_chunk_size, n_embd]);
+        native.wgpt_transpose(n_embd, vocab_chunk_size, chunkBuffer.handle, chunkBuffer.rows.handle);
+      }
+      const valid = Math.min(vocab_chunk_size, vocab_size - i * vocab_chunk_size);
+      if (valid <= 0) break;
+      const chunkResultBuffer = this.initResultBuffer([valid]);
+      passes.push(compute("wgpt_deembed", n_embd, valid, seq_length, embedBuffer.handle, chunkBuffer.rows.handle, chunkResultBuffer.handle));
+      passes.push({ flag: "copy", src: chunkResultBuffer, srcOffset: 0, dst: resultBuffer, dstOffset: 4 * i * vocab_chunk_size, size: 4 * valid });
+    }
+    return { resultBuffer, passes };
   }
 }
 

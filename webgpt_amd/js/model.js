@@ -108,6 +108,17 @@ class GPT {
   }
 
   async run(idx) {
+    if (this.externalBuffer) {
+      // model.js:211-222: the residual stream after the last layer, [seq_length, n_embd], is copied into the buffer a
+      // visualisation registered (visuals.js:48-50). The rows of the whole window are needed, so the window is
+      // recomputed, as the reference recomputes it for every token.
+      const lg = native.prefill(this.model.handle, Int32Array.from(idx), this.params.vocab_size);
+      this._history = Array.from(idx);
+      this.lastGpuMs = native.modelLastGpuMs(this.model.handle);
+      if (this.bufferSize(idx.length, this.params.n_embd) > this.externalBuffer.size) throw new Error("externalBuffer is smaller than [seq_length, n_embd]");
+      this.externalBuffer.upload(native.modelTap(this.model.handle, "residual", idx.length * this.params.n_embd));
+      return lg;
+    }
     const h = this._history;
     const extends1 = h.length > 0 && idx.length === h.length + 1 && idx.length <= this.params.n_ctx && h.every((t, i) => t === idx[i]);
     let logits;
@@ -143,7 +154,8 @@ class GPT {
 
   // The reference's pass list (model.js:118-240) built block by block from separately
   // uploaded weights and replayed through the per-block entry points.
-  async runBlocks(idx, weights) {
+  // `vocab` (optional) passes the table as the reference holds it: { vocab_chunk_size, embdBuffers, deEmbeddingsBuffers }.
+  async runBlocks(idx, weights, vocab) {
     const { n_embd, n_head, head_size, n_layer, vocab_size, hidden_size, attention_scale } = this.params;
     const seq_length = idx.length;
     const passesAll = [];
@@ -152,7 +164,9 @@ class GPT {
       passesAll.push(...passes);
       return resultBuffer;
     };
-    intermediateBuffer = residualBuffer = push(G.EmbedBlock.newInstance(idx, seq_length, n_embd, vocab_size, [weights.wte], weights.wpe, G.ResidualBlock));
+    const chunkSize = vocab ? vocab.vocab_chunk_size : vocab_size;
+    const embdBuffers = vocab ? vocab.embdBuffers : [weights.wte], deEmbeddingsBuffers = vocab ? vocab.deEmbeddingsBuffers : [weights.wte];
+    intermediateBuffer = residualBuffer = push(G.EmbedBlock.newInstance(idx, seq_length, n_embd, chunkSize, embdBuffers, weights.wpe, G.ResidualBlock));
     for (let i = 0; i < n_layer; i++) {
       const b = weights.layers[i];
       intermediateBuffer = push(G.LayerNormBlock.newInstance(seq_length, n_embd, intermediateBuffer, b.normAttentionGammaBuffer, b.normAttentionBetaBuffer));
@@ -170,7 +184,7 @@ class GPT {
       passesAll.push({ flag: "copy", src: intermediateBuffer, srcOffset: 0, dst: this.externalBuffer, dstOffset: 0, size: this.bufferSize(seq_length, n_embd) });
     }
     intermediateBuffer = push(G.LayerNormBlock.newInstance(seq_length, n_embd, intermediateBuffer, weights.normGammaBuffer, weights.normBetaBuffer));
-    const resultBuffer = push(G.DeEmbedBlock.newInstance(n_embd, vocab_size, vocab_size, seq_length, vocab_size, intermediateBuffer, [weights.wte]));
+    const resultBuffer = push(G.DeEmbedBlock.newInstance(n_embd, vocab_size, chunkSize * deEmbeddingsBuffers.length, seq_length, chunkSize, intermediateBuffer, deEmbeddingsBuffers));
     runPasses(passesAll);
     const out = resultBuffer.download();
     G.clearOperationCache();

@@ -263,6 +263,16 @@ class GPT:
         """Logits of the last token of window `idx` (model.js:104). Served from the KV
         cache when `idx` extends the previous window by one token, else recomputed."""
         idx = [int(t) for t in idx]
+        if self.externalBuffer is not None:
+            # model.js:211-222: the residual stream after the last layer, [seq_length, n_embd], is copied into the
+            # buffer a visualisation registered (visuals.js:48-50). The rows of the whole window are needed, so the
+            # window is recomputed, as the reference recomputes it for every token.
+            logits = self.prefill(idx)
+            rows = self.tap("residual", len(idx))
+            if self.bufferSize(len(idx), self.params["n_embd"]) > self.externalBuffer.size:
+                raise ValueError("externalBuffer is smaller than [seq_length, n_embd]")
+            self.externalBuffer.upload(rows)
+            return logits
         if len(idx) == len(self._history) + 1 and len(idx) <= self.params["n_ctx"] and idx[:-1] == self._history \
                 and len(self._history) > 0:
             return self.decode(idx[-1])
