@@ -71,8 +71,9 @@ int wgpt_sync(void);
  * and K % 4 == 0 (vec4 view, 219-220). bias = 0 adds none. */
 int wgpt_matmul_bias(int M, int N, int K, wgpt_buf A, wgpt_buf W, wgpt_buf bias, wgpt_buf C);
 
-/* wgpt_matmul_bias for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arithmetic and result as
+/* wgpt_matmul_bias for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, code that runs while another stream of the process is under HIP graph capture; the call itself
+ * launches on the library's own stream). It has no counterpart in the reference. Same arithmetic and result as
  * wgpt_matmul_bias for M <= 4 (the batch-1 matrix-vector product), but the ceil(K/64) * M * N partial sums live
  * in a fixed 4 MiB array inside the library's code object (one copy per GPU, held until the process ends)
  * instead of a grow-only hipMalloc: the call allocates and frees nothing. Fails with WGPT_ERR_ARG when M > 4 or

@@ -283,6 +283,24 @@ def test_persistent_decode_across_the_short_context_limit(device, name, n_layer)
     gpt.unloadBuffers()
 
 
+def test_model_create_refuses_what_the_decode_kernels_cannot_stage(device):
+    # the reference's load checks (model.js:294-297) and the library's own limits, before any tensor is uploaded
+    def create(**kw):
+        p = dict(n_layer=1, n_head=2, n_embd=128, n_ctx=16, vocab_size=40, weight_dtype=0, max_prefill=0, flags=0)
+        p.update(kw)
+        h = C.c_uint64(0)
+        _lib.call("wgpt_model_create", C.byref(_lib.Params(**p)), C.byref(h))
+        _lib.call("wgpt_model_destroy", h.value)
+    create()
+    create(n_head=48, n_embd=3072)
+    with pytest.raises(WgptError, match="n_embd above 3072"):
+        create(n_head=49, n_embd=3136)
+    with pytest.raises(WgptError, match="n_embd must be divisible by n_head"):
+        create(n_head=3, n_embd=128)
+    with pytest.raises(WgptError, match="head size above 256"):
+        create(n_head=1, n_embd=512)
+
+
 def test_external_buffer_receives_the_last_residual_rows(device):
     # model.js:211-222: with GPT.externalBuffer set (visuals.js:48-50) run() copies the residual stream after the
     # last layer, [seq_length, n_embd], into it

@@ -1065,6 +1065,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // Launches of several steps keep the first LROWS rows of the workgroup's run of the vocabulary table here
   // from start to end: that share of the table is read from memory once per launch instead of once per token.
   constexpr int LROWS = table_rows_in_lds<C>(), LR = LROWS / NW;
+  // the host takes the last step's logits from its pinned buffer for exactly these shapes (persistent_writes_host_logits),
+  // and the kernel writes them there only where it keeps table rows: the two must not drift apart
+  static_assert((LROWS > 0) == (!I8 && D <= PD_NARROW_D), "host-side and kernel-side conditions for host logits differ");
+  static_assert(LROWS == 0 || (PD_GRID * 4 * D >= 50257 && XS1 >= 4 * D), "a workgroup's run of logits is staged in the hidden row's buffer");
   float* vres = lds + lds_floats<C>();  // [LROWS * D]
 
   const int wg = blockIdx.x, tid = threadIdx.x, lane = tid & 63;

@@ -587,6 +587,8 @@ int wgpt_model_create(const wgpt_params* p, wgpt_model* out) {
   if ((p->n_embd / p->n_head) % 4 != 0) return fail(WGPT_ERR_ARG, "Model load failed: n_embd / n_head must be divisible by 4.");
   if (p->n_embd % 8 != 0) return fail(WGPT_ERR_ARG, "Cols must be divisible by 16.");  // FastMatMul on [*, n_embd]
   if (p->n_embd / p->n_head > 256) return fail(WGPT_ERR_ARG, "wgpt_model_create: head size above 256 is not supported");
+  // the decode kernels stage an input row of up to 4 n_embd floats in 48 KB of LDS
+  if (p->n_embd > 3072) return fail(WGPT_ERR_ARG, "wgpt_model_create: n_embd above 3072 is not supported");
   if (p->n_ctx > 12288) return fail(WGPT_ERR_ARG, "wgpt_model_create: n_ctx above 12288 is not supported");
   if (p->weight_dtype != 0 && p->weight_dtype != 1) return fail(WGPT_ERR_ARG, "wgpt_model_create: weight_dtype must be 0 (fp32) or 1 (int8)");
   if (p->max_prefill < 0 || p->max_prefill > p->n_ctx) return fail(WGPT_ERR_ARG, "wgpt_model_create: max_prefill must be in [0, n_ctx]");
@@ -681,6 +683,7 @@ int wgpt_prefill(wgpt_model h, const int32_t* tokens, int T, float* logits) {
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->res_host_done = m->res_host_logits = false;  // (left set by a call that failed between its launch and its read-back)
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_prefill: model not finalised");
   if (!tokens || T < 1) return fail(WGPT_ERR_ARG, "wgpt_prefill: tokens and T >= 1 required");
   if (T > m->maxT) return fail(WGPT_ERR_ARG, "wgpt_prefill: T = %d exceeds max_prefill = %d", T, m->maxT);
@@ -706,6 +709,7 @@ int wgpt_decode(wgpt_model h, int32_t token, float* logits) {
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->res_host_done = m->res_host_logits = false;  // (left set by a call that failed between its launch and its read-back)
   m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode: token id %d outside [0, %d)", token, m->V);
@@ -730,6 +734,7 @@ int wgpt_decode_greedy(wgpt_model h, int32_t token, int steps, int32_t* out_toke
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->res_host_done = m->res_host_logits = false;  // (left set by a call that failed between its launch and its read-back)
   m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_greedy: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_greedy: token id %d outside [0, %d)", token, m->V);
@@ -771,6 +776,7 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   WGPT_REQUIRE_INIT();
   Model* m = find_model(h);
   if (!m) return WGPT_ERR_ARG;
+  m->res_host_done = m->res_host_logits = false;  // (left set by a call that failed between its launch and its read-back)
   m->x_rows = 0;
   if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_decode_sample: model not finalised");
   if (token < 0 || token >= m->V) return fail(WGPT_ERR_ARG, "wgpt_decode_sample: token id %d outside [0, %d)", token, m->V);
