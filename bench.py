@@ -23,6 +23,37 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 MFMA_FP32_PEAK_FLOPS = 157.3e12  # MI355X dense fp32 matrix
 
 
+def probe_webgpu_adapter():
+    """Looks for what the reference itself would need to run on the host cores: node with a WebGPU binding
+    (the `webgpu` / `dawn.node` modules) or a Chromium that accepts --use-webgpu-adapter=swiftshader. Returns a
+    short description of what was found; nothing is installed or downloaded."""
+    import shutil
+    import subprocess
+    found = []
+    node = shutil.which("node")
+    if node:
+        for mod in ("webgpu", "dawn.node", "@webgpu/dawn"):
+            try:
+                r = subprocess.run([node, "-e", f"const m = require('{mod}'); process.exit(m ? 0 : 1)"],
+                                   capture_output=True, timeout=20)
+                if r.returncode == 0:
+                    found.append(f"node module {mod}")
+            except (OSError, subprocess.SubprocessError):
+                pass
+        try:
+            r = subprocess.run([node, "-e", "process.exit(typeof navigator !== 'undefined' && navigator.gpu ? 0 : 1)"],
+                               capture_output=True, timeout=20)
+            if r.returncode == 0:
+                found.append("navigator.gpu in node")
+        except (OSError, subprocess.SubprocessError):
+            pass
+    browsers = [b for b in ("chromium", "chromium-browser", "google-chrome", "chrome") if shutil.which(b)]
+    if found:
+        return "found, not used: " + ", ".join(found)
+    return ("none found (probed: node " + ("present" if node else "absent") + ", modules webgpu / dawn.node / @webgpu/dawn, "
+            "navigator.gpu, browsers " + (", ".join(browsers) if browsers else "none") + ")")
+
+
 def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
     """The CPU restatement of the reference's kernels (oracle/), run the way the
     reference runs: every token recomputes the whole window (model.js:69,104)."""
@@ -40,7 +71,10 @@ def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
         times.append(time.perf_counter() - t0)
         hist.append(int(np.argmax(logits)))
     ms = 1000.0 * float(np.mean(times))
+    # The reference on a CPU WebGPU adapter (Dawn/SwiftShader) is the baseline the configuration names; it is
+    # reported instead of this port only if such an adapter exists on the machine, and the line says which it was.
     return {"value": round(ms, 3), "unit": "ms/token", "cores": ref.get_threads(), "kind": "port",
+            "adapter": probe_webgpu_adapter(),
             "sample": f"{len(times)} greedy tokens after a {len(prompt)}-token prompt, whole window recomputed per "
                       f"token as GPT.run does, C restatement of the WGSL kernels with OpenMP"}
 
