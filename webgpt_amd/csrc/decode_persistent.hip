@@ -574,8 +574,12 @@ struct ItemLoader {
 #pragma unroll
       for (int cc = P::CW * H / NH; cc < P::CW * (H + 1) / NH; ++cc) {
         const int c = wave + cc * NW;
+        // (fp32 columns are only ever read under the same test, see gemv_whole / gemv_whole_ln: a column this wave
+        // does not have needs no zeros, and a dozen register moves less stand in front of the phase's dot products)
+        if constexpr (std::is_same<T, int>::value) {
 #pragma unroll
-        for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
+          for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
+        }
         if (c < (P::RAGGED ? ncols : P::CPW)) {
 #pragma unroll
           for (int seg = 0; seg < P::S; ++seg) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);

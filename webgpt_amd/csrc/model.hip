@@ -388,10 +388,10 @@ static int setup_persistent(Model* m) {
     // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
     // curves are flat within a few percent around them and over context length);
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
-    static const int tuned[5][7] = {{16, 4, 24, 96, 24, 24, 48},    // d <= 768
+    static const int tuned[5][7] = {{16, 4, 32, 80, 24, 28, 48},    // d <= 768
                                     {32, 0, 40, 96, 40, 40, 4},     // d = 1024
-                                    {20, 0, 40, 128, 24, 20, 40},   // d = 1280
-                                    {12, 12, 28, 96, 20, 12, 28},   // d = 1600, int8
+                                    {20, 0, 36, 112, 16, 16, 52},   // d = 1280
+                                    {12, 12, 20, 88, 20, 12, 44},   // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
