@@ -526,8 +526,13 @@ struct ItemLoader {
   WS& ws;
   const T* wgbase;  // this lane's word of the workgroup's first item
   int ncols, wave;
+  // int8 columns whose length is no multiple of an item's 256 rows end in an item of zeros beyond row K: its lanes
+  // beyond K request nothing (1600 rows stored as 7 items: an eighth of the bytes of such a matrix)
+  static constexpr bool TAIL = std::is_same<T, int>::value && LAYOUT == LAY_WHOLE && P::K % SEG != 0;
+  bool tail_live;   // this lane has rows of the last item
   __device__ __forceinline__ ItemLoader(WS& ws_, const T* slab, int ncols_, int wg, int wave_, int lane)
-      : ws(ws_), wgbase(slab + (size_t)wg * P::ITEMS * 64 + opaque(lane)), ncols(ncols_), wave(wave_) {}
+      : ws(ws_), wgbase(slab + (size_t)wg * P::ITEMS * 64 + opaque(lane)), ncols(ncols_), wave(wave_),
+        tail_live(!TAIL || lane * 4 < P::K - (P::S - 1) * SEG) {}
   template <int I>
   __device__ __forceinline__ void item() const {
     if constexpr (LAYOUT == LAY_WHOLE) {
@@ -537,7 +542,7 @@ struct ItemLoader {
         ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
       } else {
         zero_item(ws.w[I]);
-        if (c < (P::RAGGED ? ncols : P::CPW)) ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
+        if (c < (P::RAGGED ? ncols : P::CPW) && (!TAIL || seg != P::S - 1 || tail_live)) ws.w[I] = ld_stream(wgbase + (c * P::S + seg) * 64);
       }
     } else if constexpr (LAYOUT == LAY_RUNS) {
       // unconditional: what lies beyond the share re-reads its last item and is never used
@@ -582,7 +587,8 @@ struct ItemLoader {
         }
         if (c < (P::RAGGED ? ncols : P::CPW)) {
 #pragma unroll
-          for (int seg = 0; seg < P::S; ++seg) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);
+          for (int seg = 0; seg < P::S; ++seg)
+            if (!TAIL || seg != P::S - 1 || tail_live) ws.w[cc * P::S + seg] = ld_stream(wgbase + (c * P::S + seg) * 64);
         }
       }
     } else if constexpr (LAYOUT == LAY_RUNS) {
