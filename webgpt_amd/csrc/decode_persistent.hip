@@ -579,12 +579,8 @@ struct ItemLoader {
 #pragma unroll
       for (int cc = P::CW * H / NH; cc < P::CW * (H + 1) / NH; ++cc) {
         const int c = wave + cc * NW;
-        // (fp32 columns are only ever read under the same test, see gemv_whole / gemv_whole_ln: a column this wave
-        // does not have needs no zeros, and a dozen register moves less stand in front of the phase's dot products)
-        if constexpr (std::is_same<T, int>::value) {
 #pragma unroll
-          for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
-        }
+        for (int seg = 0; seg < P::S; ++seg) zero_item(ws.w[cc * P::S + seg]);
         if (c < (P::RAGGED ? ncols : P::CPW)) {
 #pragma unroll
           for (int seg = 0; seg < P::S; ++seg)
@@ -1042,11 +1038,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // hidden row and attention slices exchanged as words of three values (the fp32 d = 1600 shape, which lives on spilled
   // registers, spills five times as much with them and keeps {value, epoch} pairs)
   constexpr bool TRIPLE_H = I8 || D < 1600, TRIPLE_ATT = TRIPLE_H;
-  // Cached keys and values requested at the start of c_attn's phase instead of after its publish. Measured and off:
-  // the attention starts 0.2 us earlier (after the publish the rows, not q, set its start), but the requests of all
-  // 256 workgroups in front of the dot products cost more: 117M 0.1430 against 0.1396 ms/token, 345M 0.379 against 0.368,
-  // each with its poll delays re-tuned.
-  constexpr bool KV_EARLY = false;
   constexpr bool LNEPI = FOLD && LN_EPILOGUE && D <= 1280;  // (the fp32 d = 1600 shape, short of registers, spills six times as much with it)  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln)
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
@@ -1211,24 +1202,6 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         }
         wait_loads();
         TRACE(1 + li * 8 + PH);
-        if constexpr (KV_EARLY) {
-          // This layer's cached keys and values of the slice, a whole phase before the attention needs them: they
-          // come from memory in 0.5-0.8 us, and requested after the publish they, not q, set the attention's start.
-          // No branch around the loads (the compiler would wait for them where its arms join): workgroups without
-          // the attention role, and lanes without a row, read one row of the positional table instead, finite values
-          // that a score of -inf multiplies by zero. (Ordinary loads: a cached row never changes once written and is
-          // only requested below the position, see the end-of-token exchange.)
-          const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
-#pragma unroll
-          for (int i = 0; i < MAXKV; ++i) {
-            const int j = c0 + g16 + 32 * i;
-            const bool row = att_role && i < nkv && j < c1 && j < pos;
-            const float* kp = row ? Kc + (size_t)j * HS + sub * 4 : a.wpe + sub * 4;
-            const float* vp = row ? Vc + (size_t)j * HS + sub * 4 : a.wpe + sub * 4;
-            kreg[i] = *reinterpret_cast<const float4*>(kp);
-            vreg[i] = *reinterpret_cast<const float4*>(vp);
-          }
-        }
         const LoadC nextC(wY, slab + a.slab_offC, ncC, wg, wave, lane);
         if (DUAL && !SPREAD) nextC.early();
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
@@ -1246,7 +1219,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         if (!DUAL) nextC.all();
         else if (!SPREAD) nextC.late();
         TRACE5(5);
-        if (!KV_EARLY && att_role) {
+        if (att_role) {
           // this layer's cached keys and values of the slice
           const int g16 = opaque(tid >> 4), sub = opaque(tid & 15);
 #pragma unroll
