@@ -125,6 +125,9 @@ def main():
                     help="prompt length (default: the configuration's); the decode steps that follow must fit n_ctx")
     ap.add_argument("--mode", type=int, default=None, help="decode implementation (default: library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tune-delays", type=int, default=0, metavar="ROUNDS",
+                    help="before anything is timed, search the persistent kernel's poll delays on this GPU "
+                         "(wgpt_model_tune_poll_delays) with this many passes")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run three 256 MiB device-to-device copies (a kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -162,6 +165,15 @@ def main():
     gpt.initialize()
     if args.mode is not None:
         gpt.set_decode_mode(args.mode)
+    tuned = None
+    if args.tune_delays > 0 and args.mode in (None, 1):
+        try:
+            t0 = time.perf_counter()
+            row, before, after = gpt.tune_poll_delays(args.tune_delays)
+            tuned = {"delays": row, "ms_per_token_before": round(before, 5), "ms_per_token_after": round(after, 5),
+                     "search_s": round(time.perf_counter() - t0, 2)}
+        except WgptError as e:
+            tuned = {"error": str(e)}
 
     # prefill (untimed for the headline; reported separately)
     gpt.prefill(prompt)  # first call also loads the code objects
@@ -247,6 +259,11 @@ def main():
                              "up to a third of the vocabulary table in LDS and registers and reads that much less per step), "
                              "null where no counter run exists for the configuration"},
     }
+    if persistent:
+        try:
+            out["poll_delays"] = {"in_use": gpt.poll_delays(), "tuned_on_this_gpu": tuned}
+        except WgptError:
+            pass
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, tensors, prompt)
     gpt.unloadBuffers()

@@ -129,7 +129,8 @@ typedef struct {
 } wgpt_params;
 
 enum {
-  WGPT_FLAG_TAPS = 1 /* keep the activation taps of the last wgpt_prefill for wgpt_model_tap */
+  WGPT_FLAG_TAPS = 1, /* keep the activation taps of the last wgpt_prefill for wgpt_model_tap */
+  WGPT_FLAG_TUNE_DELAYS = 2 /* wgpt_model_finalize ends with wgpt_model_tune_poll_delays(m, 2, ...) */
 };
 
 int wgpt_model_create(const wgpt_params* params, wgpt_model* out);
@@ -184,6 +185,17 @@ int wgpt_model_decode_bytes(wgpt_model m, int t, uint64_t* bytes);
 /* Selects the decode implementation: 0 = one kernel per block, 1 = persistent
  * whole-token kernel. Default is the fastest available. */
 int wgpt_model_set_decode_mode(wgpt_model m, int mode);
+/* The persistent decode kernel waits a fixed time after publishing before it first looks for the other workgroups'
+ * values (seven delays, one per exchange; a table per model width is built in, measured on one MI355X). This searches
+ * around the current row on the GPU the model lives on: `rounds` passes of coordinate descent (0 = only measure), each
+ * candidate timed with multi-step launches at a mid-length context, the found row kept only if it beats the starting
+ * one by more than the run-to-run noise when the two are timed alternately. Needs position 0 (before the first
+ * prefill, or after wgpt_model_reset_cache); it overwrites key/value rows that every later call rewrites before
+ * reading. chosen[7], ms_before, ms_after (milliseconds per token of the starting and the kept row) may be NULL.
+ * No counterpart in the reference (its dispatches are ordered by the WebGPU queue). About a second for GPT-2 117M. */
+int wgpt_model_tune_poll_delays(wgpt_model m, int rounds, int32_t* chosen, float* ms_before, float* ms_after);
+/* The seven delays in use (units of 64 clocks), out[7]. */
+int wgpt_model_poll_delays(wgpt_model m, int32_t* out);
 int wgpt_model_destroy(wgpt_model m);
 
 /* ---- synthetic tensors (host only, no device needed): the seeded generator the

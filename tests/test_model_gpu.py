@@ -201,6 +201,37 @@ def test_persistent_decode_matches_per_block_decode_and_oracle(device, name, ste
     gpt.unloadBuffers()
 
 
+def test_poll_delay_search_changes_timing_only(device):
+    # wgpt_model_tune_poll_delays: the row it keeps is no slower than the one it started from (as it measured them),
+    # logits and greedy ids of a context decoded afterwards are those of a model that never searched, and it refuses
+    # to run while a context is in use
+    cfg = dict(synth.CONFIGS["toy"])
+    gpt, tensors = load(cfg, seed=5)
+    tokens = synth.tokens(8, "prompt", 12, cfg["vocab_size"])
+    lg = gpt.prefill(tokens)
+    want_ids = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), 30)]
+    gpt.prefill(tokens[:11])
+    want_logits = gpt.decode(int(tokens[11]))
+    with pytest.raises(WgptError, match="context is in use"):
+        gpt.tune_poll_delays(1)
+    _lib.call("wgpt_model_reset_cache", gpt._handle)
+    start = gpt.poll_delays()
+    row, before, after = gpt.tune_poll_delays(1)
+    print("poll delays", start, "->", row, "ms/token", before, "->", after)
+    assert len(row) == 7 and all(0 <= v <= 1024 for v in row) and row == gpt.poll_delays()
+    assert 0 < after <= before
+    lg = gpt.prefill(tokens)
+    assert [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), 30)] == want_ids
+    gpt.prefill(tokens[:11])
+    assert np.array_equal(gpt.decode(int(tokens[11])), want_logits)
+    gpt.unloadBuffers()
+    # the same search as the last step of wgpt_model_finalize
+    gpt2, _ = load(cfg, seed=5, flags=_lib.FLAG_TUNE_DELAYS)
+    lg = gpt2.prefill(tokens)
+    assert [int(t) for t in gpt2.decode_greedy(int(np.argmax(lg)), 30)] == want_ids
+    gpt2.unloadBuffers()
+
+
 @pytest.mark.parametrize("name", ["gpt2-345m", "gpt2-774m"])
 def test_larger_shapes_decode_against_oracle(device, name):
     # the persistent decode kernel is instantiated per model width; check the other widths too

@@ -25,6 +25,7 @@ class Params(C.Structure):
 
 
 FLAG_TAPS = 1
+FLAG_TUNE_DELAYS = 2
 
 _u64 = C.c_uint64
 _sz = C.c_size_t
@@ -72,6 +73,8 @@ _SIGNATURES = {
     "wgpt_model_last_gpu_ms": ([_u64, _fp], True),
     "wgpt_model_decode_bytes": ([_u64, _int, C.POINTER(_u64)], True),
     "wgpt_model_set_decode_mode": ([_u64, _int], True),
+    "wgpt_model_tune_poll_delays": ([_u64, _int, _ip, _fp, _fp], True),
+    "wgpt_model_poll_delays": ([_u64, _ip], True),
     "wgpt_model_destroy": ([_u64], True),
     "wgpt_synth_normal": ([C.c_uint32, C.c_uint32, _sz, C.c_double, _fp], False),
     "wgpt_synth_tokens": ([C.c_uint32, C.c_uint32, _sz, C.c_uint32, _ip], False),

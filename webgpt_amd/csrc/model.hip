@@ -387,11 +387,12 @@ static int setup_persistent(Model* m) {
   {
     // measured optima on MI355X (coordinate descent on ms/token at contexts of 130-770; the
     // curves are flat within a few percent around them and over context length);
-    // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for tuning
+    // wgpt_model_tune_poll_delays searches around them on the GPU at hand,
+    // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for experiments
     static const int tuned[5][7] = {{16, 4, 32, 80, 24, 28, 48},    // d <= 768
-                                    {32, 0, 40, 96, 40, 40, 4},     // d = 1024
-                                    {20, 0, 36, 112, 16, 16, 52},   // d = 1280
-                                    {12, 12, 20, 88, 20, 12, 44},   // d = 1600, int8
+                                    {36, 0, 32, 104, 40, 40, 4},    // d = 1024
+                                    {20, 0, 36, 128, 16, 16, 52},   // d = 1280
+                                    {12, 12, 28, 104, 20, 12, 44},  // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
     const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
@@ -676,6 +677,7 @@ int wgpt_model_finalize(wgpt_model h) {
   m->decode_mode = m->persist_ok ? 1 : 0;
   m->pos = 0;
   m->finalized = true;
+  if ((m->p.flags & WGPT_FLAG_TUNE_DELAYS) && m->persist_ok) return wgpt_model_tune_poll_delays(h, 2, nullptr, nullptr, nullptr);
   return WGPT_OK;
 }
 
@@ -829,6 +831,138 @@ int wgpt_decode_sample(wgpt_model h, int32_t token, int steps, int top_k, double
   }
   if (persistent && (rc = check_persistent(m))) return rc;
   m->pos = pos_before + steps;
+  return WGPT_OK;
+}
+
+// One timed launch of `steps` greedy steps from position p0 (token 0), for the delay search: GPU milliseconds, or a
+// negative value when the launch failed. The key/value rows it writes are rows that every later call writes before it
+// reads them (a model's position is 0 while this runs).
+static float timed_trial(Model* m, int p0, int steps) {
+  m->pos = p0;
+  if (hipEventRecord(m->ev0, rt().stream) != hipSuccess) return -1.f;
+  if (decode_persistent(m, steps, 1, 1.0, nullptr, 0, false) != WGPT_OK) return -1.f;
+  if (hipEventRecord(m->ev1, rt().stream) != hipSuccess) return -1.f;
+  if (hipMemcpyAsync(&m->pin[1], m->perr, sizeof(int), hipMemcpyDeviceToHost, rt().stream) != hipSuccess) return -1.f;
+  if (hipStreamSynchronize(rt().stream) != hipSuccess) return -1.f;
+  m->pos = 0;
+  if (m->pin[1] != 0) return -1.f;
+  float ms = -1.f;
+  if (hipEventElapsedTime(&ms, m->ev0, m->ev1) != hipSuccess) return -1.f;
+  return ms;
+}
+
+int wgpt_model_tune_poll_delays(wgpt_model h, int rounds, int32_t* chosen, float* ms_before, float* ms_after) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m) return WGPT_ERR_ARG;
+  if (!m->finalized) return fail(WGPT_ERR_STATE, "wgpt_model_tune_poll_delays: model not finalised");
+  if (!m->persist_ok || m->decode_mode != 1)
+    return fail(WGPT_ERR_STATE, "wgpt_model_tune_poll_delays: the persistent decode kernel is not in use for this model");
+  if (m->pos != 0) return fail(WGPT_ERR_STATE, "wgpt_model_tune_poll_delays: a context is in use (position %d); call it before the first prefill or after wgpt_model_reset_cache", m->pos);
+  if (rounds < 0 || rounds > 8) return fail(WGPT_ERR_ARG, "wgpt_model_tune_poll_delays: rounds must be in [0, 8]");
+  m->res_host_done = m->res_host_logits = false;
+  m->x_rows = 0;
+  // a trial is two launches, at three tenths and at three quarters of the context (the attention exchange's best
+  // delays move with the context length: a row found at one length loses at another), together long enough (about
+  // 5 ms) that the event clock's granularity does not matter
+  const int pa = m->ctx * 3 / 10, pb = m->ctx * 3 / 4;
+  int steps = m->ctx - pb < 8 ? m->ctx - pb : 8;
+  if (steps < 1 || pa < 1) return fail(WGPT_ERR_STATE, "wgpt_model_tune_poll_delays: context too short");
+  const auto timed_pair = [&](int n) {
+    const float a = timed_trial(m, pa, n);
+    if (a < 0) return -1.f;
+    const float b = timed_trial(m, pb, n);
+    return b < 0 ? -1.f : a + b;
+  };
+  const auto failed = [&](const int* restore) -> int {
+    for (int i = 0; i < 7; ++i) m->pa.delay[i] = restore[i];
+    m->pos = 0;
+    if (m->pin[1] != 0) { (void)check_persistent(m); return WGPT_ERR_DEVICE; }
+    return fail(WGPT_ERR_DEVICE, "wgpt_model_tune_poll_delays: a trial launch failed");
+  };
+  int start[7];
+  for (int i = 0; i < 7; ++i) start[i] = m->pa.delay[i];
+  float t = timed_pair(steps);
+  if (t < 0) return failed(start);
+  {
+    const float per_step = t / (2 * steps);
+    int want = per_step > 0 ? (int)(2.5f / per_step) : 32;
+    want = want < 8 ? 8 : (want > 32 ? 32 : want);
+    steps = m->ctx - pb < want ? m->ctx - pb : want;
+    if (pb - pa < steps) steps = pb - pa;
+  }
+  const auto measure = [&](int reps) {
+    float best = 1e30f;
+    for (int r = 0; r < reps; ++r) {
+      const float v = timed_pair(steps);
+      if (v < 0) return -1.f;
+      best = v < best ? v : best;
+    }
+    return best;
+  };
+  const float before = measure(5);
+  if (before < 0) return failed(start);
+  // coordinate descent, the delays with the steepest curves first; a move must gain more than the run-to-run noise
+  static const int order[7] = {3, 2, 0, 4, 5, 6, 1};
+  static const int moves[4] = {-8, -4, 4, 8};
+  float cur = before;
+  for (int round = 0; round < rounds; ++round) {
+    bool moved = false;
+    for (int oi = 0; oi < 7; ++oi) {
+      const int c = order[oi];
+      const int here = m->pa.delay[c];
+      cur = measure(3);
+      if (cur < 0) return failed(start);
+      int best_v = here;
+      float best_t = cur * 0.997f;
+      for (int mv : moves) {
+        const int v = here + mv;
+        if (v < 0 || v > 1024) continue;
+        m->pa.delay[c] = v;
+        const float tv = measure(3);
+        if (tv < 0) return failed(start);
+        if (tv < best_t) { best_t = tv; best_v = v; }
+      }
+      m->pa.delay[c] = best_v;
+      moved = moved || best_v != here;
+    }
+    if (!moved) break;
+  }
+  // the found row against the starting one, alternating: kept only when it wins by more than the noise
+  int found[7];
+  bool differs = false;
+  for (int i = 0; i < 7; ++i) { found[i] = m->pa.delay[i]; differs = differs || found[i] != start[i]; }
+  float t_start = before, t_found = before;
+  if (differs) {
+    t_start = t_found = 1e30f;
+    for (int r = 0; r < 4; ++r) {
+      for (int i = 0; i < 7; ++i) m->pa.delay[i] = start[i];
+      float v = measure(2);
+      if (v < 0) return failed(start);
+      t_start = v < t_start ? v : t_start;
+      for (int i = 0; i < 7; ++i) m->pa.delay[i] = found[i];
+      v = measure(2);
+      if (v < 0) return failed(start);
+      t_found = v < t_found ? v : t_found;
+    }
+    if (!(t_found < t_start * 0.995f)) {
+      for (int i = 0; i < 7; ++i) m->pa.delay[i] = start[i];
+      t_found = t_start;
+    }
+  }
+  m->pos = 0;
+  if (chosen) for (int i = 0; i < 7; ++i) chosen[i] = m->pa.delay[i];
+  if (ms_before) *ms_before = t_start / (2 * steps);
+  if (ms_after) *ms_after = t_found / (2 * steps);
+  return WGPT_OK;
+}
+
+int wgpt_model_poll_delays(wgpt_model h, int32_t* out) {
+  WGPT_REQUIRE_INIT();
+  Model* m = find_model(h);
+  if (!m || !out) return fail(WGPT_ERR_ARG, "wgpt_model_poll_delays: NULL argument");
+  if (!m->finalized || !m->persist_ok) return fail(WGPT_ERR_STATE, "wgpt_model_poll_delays: the persistent decode kernel is not set up for this model");
+  for (int i = 0; i < 7; ++i) out[i] = m->pa.delay[i];
   return WGPT_OK;
 }
 

@@ -30,7 +30,8 @@ void* g_lib = nullptr;
   X(wgpt_model_reset_cache) X(wgpt_model_position) X(wgpt_model_tap) X(wgpt_model_last_gpu_ms)          \
   X(wgpt_model_decode_bytes) X(wgpt_model_set_decode_mode) X(wgpt_model_destroy) X(wgpt_synth_normal)   \
   X(wgpt_synth_tokens) X(wgpt_synth_int8_packed) X(wgpt_synth_uniform) X(wgpt_synth_tensor_id)   \
-  X(wgpt_decode_sample) X(wgpt_sample_topk) X(wgpt_matmul_bias_noalloc) X(wgpt_softmax_t) X(wgpt_transpose)
+  X(wgpt_decode_sample) X(wgpt_sample_topk) X(wgpt_matmul_bias_noalloc) X(wgpt_softmax_t) X(wgpt_transpose)   \
+  X(wgpt_model_tune_poll_delays) X(wgpt_model_poll_delays)
 
 #define DECL(name) decltype(&::name) p_##name = nullptr;
 WGPT_FUNCS(DECL)
@@ -235,6 +236,38 @@ FN(ModelPosition) { Args a(env, info); uint64_t m = a.u64(0); if (!a.ok) return 
 FN(ModelLastGpuMs) { Args a(env, info); uint64_t m = a.u64(0); if (!a.ok) return nullptr; float ms = 0; if (failed(env, p_wgpt_model_last_gpu_ms(m, &ms))) return nullptr; return number(env, ms); }
 FN(ModelDecodeBytes) { Args a(env, info); uint64_t m = a.u64(0); int t = a.i32(1); if (!a.ok) return nullptr; uint64_t b = 0; if (failed(env, p_wgpt_model_decode_bytes(m, t, &b))) return nullptr; return number(env, (double)b); }
 
+// seven poll delays (and, after a search, the milliseconds per token before and after it) as a Float32Array
+FN(ModelPollDelays) {  // (model) -> Float32Array[7]
+  Args a(env, info);
+  uint64_t m = a.u64(0);
+  if (!a.ok) return nullptr;
+  int32_t row[7];
+  if (failed(env, p_wgpt_model_poll_delays(m, row))) return nullptr;
+  napi_value ab, ta;
+  void* p;
+  if (napi_create_arraybuffer(env, 7 * sizeof(float), &p, &ab) != napi_ok) return nullptr;
+  napi_create_typedarray(env, napi_float32_array, 7, ab, 0, &ta);
+  for (int i = 0; i < 7; ++i) ((float*)p)[i] = (float)row[i];
+  return ta;
+}
+FN(ModelTunePollDelays) {  // (model, rounds) -> Float32Array[9]: the row kept, ms/token before, ms/token after
+  Args a(env, info);
+  uint64_t m = a.u64(0);
+  int rounds = a.i32(1);
+  if (!a.ok) return nullptr;
+  int32_t row[7];
+  float before = 0, after = 0;
+  if (failed(env, p_wgpt_model_tune_poll_delays(m, rounds, row, &before, &after))) return nullptr;
+  napi_value ab, ta;
+  void* p;
+  if (napi_create_arraybuffer(env, 9 * sizeof(float), &p, &ab) != napi_ok) return nullptr;
+  napi_create_typedarray(env, napi_float32_array, 9, ab, 0, &ta);
+  for (int i = 0; i < 7; ++i) ((float*)p)[i] = (float)row[i];
+  ((float*)p)[7] = before;
+  ((float*)p)[8] = after;
+  return ta;
+}
+
 napi_value new_f32(napi_env env, size_t count, float** data) {
   napi_value ab, ta;
   void* p;
@@ -398,6 +431,7 @@ napi_value InitModule(napi_env env, napi_value exports) {
       {"modelCreate", ModelCreate}, {"modelSetTensor", ModelSetTensor}, {"modelFinalize", ModelFinalize},
       {"modelDestroy", ModelDestroy}, {"modelResetCache", ModelResetCache}, {"modelSetDecodeMode", ModelSetDecodeMode},
       {"modelPosition", ModelPosition}, {"modelLastGpuMs", ModelLastGpuMs}, {"modelDecodeBytes", ModelDecodeBytes},
+      {"modelPollDelays", ModelPollDelays}, {"modelTunePollDelays", ModelTunePollDelays},
       {"prefill", Prefill}, {"decode", Decode}, {"decodeGreedy", DecodeGreedy}, {"decodeSample", DecodeSample}, {"sampleTopK", SampleTopK}, {"modelTap", ModelTap},
       {"synthNormal", SynthNormal}};
   for (const auto& e : table) {

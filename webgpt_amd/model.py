@@ -296,6 +296,19 @@ class GPT:
     def set_decode_mode(self, mode):
         _lib.call("wgpt_model_set_decode_mode", self._handle, int(mode))
 
+    def tune_poll_delays(self, rounds=2):
+        """Searches the persistent decode kernel's seven poll delays on this GPU (wgpt_model_tune_poll_delays; needs
+        position 0). Returns (delays, ms_per_token_before, ms_per_token_after)."""
+        chosen = (C.c_int32 * 7)()
+        before, after = C.c_float(0), C.c_float(0)
+        _lib.call("wgpt_model_tune_poll_delays", self._handle, int(rounds), chosen, C.byref(before), C.byref(after))
+        return [int(v) for v in chosen], before.value, after.value
+
+    def poll_delays(self):
+        out = (C.c_int32 * 7)()
+        _lib.call("wgpt_model_poll_delays", self._handle, out)
+        return [int(v) for v in out]
+
     def generate(self, prompt, max_new_tokens, top_k, temperature):
         """The loop of model.js:53-102. `prompt` is a string when a tokenizer was
         given, else a list of token ids; yields decoded text or ids accordingly."""
