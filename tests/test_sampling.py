@@ -129,6 +129,36 @@ def test_decode_sample_follows_the_reference_loop(device, mode, top_k):
         gpt.unloadBuffers()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("top_k", [1, 3, 12])
+def test_generate_in_bursts_yields_the_tokens_of_a_call_per_token(device, monkeypatch, top_k):
+    """GPT.generate makes up to `burst` tokens per call once the window is cached, each with the draw the
+    reference's loop (model.js:53-102) would have made for it: same ids as one call per token, also across
+    the end of the context (sliding window) and when max_new_tokens is no multiple of the burst."""
+    import random
+    import time
+    from webgpt_amd.model import GPT
+    cfg = small_cfg(n_layer=2, n_head=6, n_embd=384, n_ctx=40, vocab_size=300)
+    tensors = make_model(cfg, 22)
+    gpt = GPT(None, "char", tensors=tensors, params=synth.model_params(cfg))
+    gpt.initialize()
+    try:
+        prompt = [int(t) for t in synth.tokens(22, "prompt", 9, cfg["vocab_size"])]
+        out, ms = {}, {}
+        for burst in (1, 8, 5):
+            gpt.burst = burst
+            random.seed(1234)
+            gpt._history = []
+            t0 = time.perf_counter()
+            out[burst] = [int(t) for t in gpt.generate(prompt, 43, top_k, 0.9)]   # runs past the 40 positions of the context
+            ms[burst] = (time.perf_counter() - t0) * 1000.0 / 43
+        print("generate ms/token by burst", {b: round(v, 4) for b, v in ms.items()})
+        assert len(out[1]) == 43
+        assert out[8] == out[1] and out[5] == out[1]
+    finally:
+        gpt.unloadBuffers()
+
+
 def _lib_error():
     from webgpt_amd import _lib
     return _lib.WgptError

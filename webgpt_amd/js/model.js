@@ -40,6 +40,7 @@ class GPT {
     this._quantize = options.quantize;  // "int8": quantise the fp32 linear weights while loading (quantize.js)
     this._history = [];
     this.lastGpuMs = 0;
+    this.burst = options.burst || 8;  // tokens generate() makes per call once the window is cached (1: a call per token)
   }
 
   async initialize() {
@@ -91,8 +92,22 @@ class GPT {
       if (cached && top_k >= 1 && top_k <= 1024 && temperature > 0) {
         // the window extends the cached one by a token: that token goes in, the next one is selected
         // on the device (selectTopK, cpuSoftmax, sampleFromDistribution with this Math.random() draw)
-        // and the logits are never read back
-        idx_next = this.decodeSample(idx_cond[idx_cond.length - 1], top_k, temperature, [Math.random()])[0];
+        // and the logits are never read back. Up to `burst` tokens are made by one call, each with the
+        // draw the reference's loop would have made for it (one Math.random() per token, in order); they
+        // are yielded one by one. burst = 1 is a call per token.
+        const room = this.params.n_ctx - h.length;  // positions the cache still has
+        const steps = Math.max(1, Math.min(this.burst | 0, max_new_tokens - i, room));
+        const draws = [];
+        for (let k = 0; k < steps; k++) draws.push(Math.random());
+        const ids = this.decodeSample(idx_cond[idx_cond.length - 1], top_k, temperature, draws);
+        const lapsed = (performance.now() - startTime) / steps;
+        for (let k = 0; k < steps; k++) {
+          i + k >= warmupRuns && (totalTime += lapsed);
+          history = history.concat(ids[k]);
+          yield this.tokenizer ? this.tokenizer.decode([ids[k]]) : ids[k];
+        }
+        i += steps - 1;
+        continue;
       } else {
         const logits = await this.run(idx_cond);
         const { topKIndices, topKProbs } = G.selectTopK(logits, top_k);

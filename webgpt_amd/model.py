@@ -97,6 +97,7 @@ class GPT:
         self._quantize = quantize
         self._handle = None
         self._history = []
+        self.burst = 8  # tokens generate() makes per call once the window is cached (1: a call per token)
         self.lastGpuMs = 0.0
 
     # ---------------- lifecycle ----------------
@@ -319,24 +320,37 @@ class GPT:
         warmupRuns = 3
         totalTime = 0.0
         n_ctx = self.params["n_ctx"]
-        for i in range(max_new_tokens):
+        i = 0
+        while i < max_new_tokens:
             idx_cond = history[-n_ctx:]
             startTime = time.perf_counter()
             h = self._history
             cached = len(h) > 0 and len(idx_cond) == len(h) + 1 and len(idx_cond) <= n_ctx and idx_cond[:-1] == h
             if cached and 1 <= top_k <= 1024 and temperature > 0:
                 # the window extends the cached one by a token: that token goes in, the next one is
-                # selected on the device with this draw, and the logits are never read back
-                idx_next = int(self.decode_sample(idx_cond[-1], 1, top_k, temperature, [random.random()])[0])
-            else:
-                logits = self.run(idx_cond)
-                sel = sampling.selectTopK(logits, top_k) if top_k != 1 else \
-                    {"topKIndices": [int(np.argmax(logits))], "topKProbs": [float(np.max(logits))]}
-                probs = sampling.cpuSoftmax(sel["topKProbs"], temperature)
-                idx_next = sel["topKIndices"][sampling.sampleFromDistribution(probs)]
+                # selected on the device with this draw, and the logits are never read back. Up to
+                # self.burst tokens are made by one call, each with the draw the reference's loop would
+                # have made for it (one per token, in order); they are yielded one by one.
+                steps = max(1, min(int(self.burst), max_new_tokens - i, n_ctx - len(h)))
+                draws = [random.random() for _ in range(steps)]
+                ids = [int(t) for t in self.decode_sample(idx_cond[-1], steps, top_k, temperature, draws)]
+                lapsed = (time.perf_counter() - startTime) * 1000.0 / steps
+                for k, t in enumerate(ids):
+                    if i + k >= warmupRuns:
+                        totalTime += lapsed
+                    history = history + [t]
+                    yield self.tokenizer.decode([t]) if self.tokenizer else t
+                i += steps
+                continue
+            logits = self.run(idx_cond)
+            sel = sampling.selectTopK(logits, top_k) if top_k != 1 else \
+                {"topKIndices": [int(np.argmax(logits))], "topKProbs": [float(np.max(logits))]}
+            probs = sampling.cpuSoftmax(sel["topKProbs"], temperature)
+            idx_next = sel["topKIndices"][sampling.sampleFromDistribution(probs)]
             lapsed = (time.perf_counter() - startTime) * 1000.0
             if i >= warmupRuns:
                 totalTime += lapsed
             history = history + [idx_next]
             yield self.tokenizer.decode([idx_next]) if self.tokenizer else idx_next
+            i += 1
         self.averageMs = totalTime / max(1, max_new_tokens - warmupRuns)
