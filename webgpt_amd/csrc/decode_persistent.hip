@@ -1038,7 +1038,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // hidden row and attention slices exchanged as words of three values (the fp32 d = 1600 shape, which lives on spilled
   // registers, spills five times as much with them and keeps {value, epoch} pairs)
   constexpr bool TRIPLE_H = I8 || D < 1600, TRIPLE_ATT = TRIPLE_H;
-  constexpr bool LNEPI = FOLD && LN_EPILOGUE && D <= 1280;  // (the fp32 d = 1600 shape, short of registers, spills six times as much with it)  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln)
+  // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln; the fp32 d = 1600
+  // shape spills six times as much with it)
+  constexpr bool LNEPI = FOLD && LN_EPILOGUE && D <= 1280;
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
   constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;  // floats of the staged exchange words
