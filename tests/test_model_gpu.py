@@ -232,6 +232,32 @@ def test_poll_delay_search_changes_timing_only(device):
     gpt2.unloadBuffers()
 
 
+@pytest.mark.parametrize("start", [2**31 - 1 - 60, 2**31 - 1 - 1000, 2**31 - 1 - 1500])
+def test_epoch_counter_restarts_below_its_limit(device, monkeypatch, start):
+    # the exchange words carry a 32-bit epoch that only grows; a model that has decoded for hours reaches the
+    # limit, clears its exchange buffers and starts over. Started just below the limit (at once, within the first
+    # greedy call, within the third), the tokens and logits are those of a counter that starts at 0.
+    cfg = dict(synth.CONFIGS["toy"])
+    cfg["n_layer"] = 3
+    tokens = synth.tokens(8, "prompt", 12, cfg["vocab_size"])
+    runs = {}
+    for s0 in (0, start):
+        if s0:
+            monkeypatch.setenv("WEBGPT_AMD_EPOCH_START", str(s0))
+        else:
+            monkeypatch.delenv("WEBGPT_AMD_EPOCH_START", raising=False)
+        gpt, _ = load(cfg, seed=5)
+        lg = gpt.prefill(tokens)
+        ids = [int(t) for t in gpt.decode_greedy(int(np.argmax(lg)), 40)]
+        ids += [int(t) for t in gpt.decode_greedy(ids[-1], 40)]
+        ids += [int(t) for t in gpt.decode_greedy(ids[-1], 40)]
+        last = gpt.decode(ids[-1])
+        runs[s0] = (ids, last.copy())
+        gpt.unloadBuffers()
+    assert runs[start][0] == runs[0][0]
+    assert np.array_equal(runs[start][1], runs[0][1])
+
+
 @pytest.mark.parametrize("name", ["gpt2-345m", "gpt2-774m"])
 def test_larger_shapes_decode_against_oracle(device, name):
     # the persistent decode kernel is instantiated per model width; check the other widths too

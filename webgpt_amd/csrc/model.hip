@@ -425,6 +425,12 @@ static int setup_persistent(Model* m) {
   WGPT_HIP(hipMemsetAsync(a.trace, 0, sizeof(unsigned long long) * 512 * G, rt().stream));
 #endif
   m->epoch = 0;
+  // WEBGPT_AMD_EPOCH_START: tests start the counter just below its limit to run the restart above
+  if (const char* e = getenv("WEBGPT_AMD_EPOCH_START")) {
+    char* end = nullptr;
+    const unsigned long v = strtoul(e, &end, 10);
+    if (end != e && v <= 0x7fffffffu) m->epoch = (unsigned)v;
+  }
   m->persist_ok = true;
   return WGPT_OK;
 }
@@ -447,8 +453,9 @@ static int decode_persistent(Model* m, int steps, int top_k = 1, double temperat
   a.temperature = temperature;
   a.u = u_dev;
   const unsigned per_step = persistent_epochs_per_step(m->L);
-  if (m->epoch > 0xffffffffu - per_step * (unsigned)steps - 8u) {
-    // epoch counter about to wrap: start over from clean exchange buffers
+  if (m->epoch > 0x7fffffffu - per_step * (unsigned)steps - 8u) {
+    // epoch counter about to leave the positive ints (the kernel's error word is the epoch of the wait that
+    // expired, as an int; negative values are its other codes): start over from clean exchange buffers
     const size_t words = (size_t)(a.bufAM + 2 * PD_TOPK * PD_GRID - a.bufQKV);
     WGPT_HIP(hipMemsetAsync(a.bufQKV, 0, words * sizeof(unsigned long long), rt().stream));
     m->epoch = 0;
