@@ -258,6 +258,36 @@ def test_epoch_counter_restarts_below_its_limit(device, monkeypatch, start):
     assert np.array_equal(runs[start][1], runs[0][1])
 
 
+def test_two_models_decode_interleaved(device):
+    # two models alive at once (their own caches, exchange buffers and epochs), their decode calls interleaved:
+    # each gives what it gives alone
+    cfg = dict(synth.CONFIGS["toy"])
+    cfg["n_layer"] = 2
+    tokens = synth.tokens(8, "prompt", 10, cfg["vocab_size"])
+    alone = {}
+    for seed in (5, 6):
+        gpt, _ = load(cfg, seed=seed)
+        lg = gpt.prefill(tokens)
+        first = int(np.argmax(lg))
+        ids = [int(t) for t in gpt.decode_greedy(first, 9)]
+        alone[seed] = (first, ids, gpt.decode(ids[-1]).copy())
+        gpt.unloadBuffers()
+    a, _ = load(cfg, seed=5)
+    b, _ = load(cfg, seed=6)
+    la, lb = a.prefill(tokens), b.prefill(tokens)
+    fa, fb = int(np.argmax(la)), int(np.argmax(lb))
+    ia, ib = [], []
+    ta, tb = fa, fb
+    for _ in range(3):   # three calls of three steps each, alternating
+        ia += [int(t) for t in a.decode_greedy(ta, 3)]
+        ib += [int(t) for t in b.decode_greedy(tb, 3)]
+        ta, tb = ia[-1], ib[-1]
+    assert (fa, ia) == alone[5][:2] and (fb, ib) == alone[6][:2]
+    assert np.array_equal(b.decode(ib[-1]), alone[6][2]) and np.array_equal(a.decode(ia[-1]), alone[5][2])
+    a.unloadBuffers()
+    b.unloadBuffers()
+
+
 @pytest.mark.parametrize("name", ["gpt2-345m", "gpt2-774m"])
 def test_larger_shapes_decode_against_oracle(device, name):
     # the persistent decode kernel is instantiated per model width; check the other widths too
