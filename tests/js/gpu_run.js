@@ -60,6 +60,23 @@ async function main() {
   let first = 0;
   for (let i = 1; i < lg.length; i++) if (lg[i] > lg[first]) first = i;
   out.greedy = [first].concat(Array.from(gpt.decodeGreedy(first, 9)));
+  // generate() with top_k = 3 and a seeded Math.random: a call per token, bursts of 8, bursts of 5 (19 tokens: no
+  // multiple of either)
+  {
+    const realRandom = Math.random;
+    out.bursts = {};
+    for (const burst of [1, 8, 5]) {
+      let state = 12345;
+      Math.random = () => { state = (state * 1103515245 + 12345) % 2147483648; return state / 2147483648; };
+      gpt.burst = burst;
+      gpt._history = [];
+      const ids = [];
+      for await (const id of gpt.generate(tokens.slice(0, 8), 19, 3, 0.9)) ids.push(id);
+      out.bursts[burst] = ids;
+    }
+    Math.random = realRandom;
+    gpt.burst = 8;
+  }
   // token selection on the device: one buffer-level call, then a sampled continuation
   const probe = new Float32Array([0.5, 2.0, -1.0, 2.0, 1.5]);
   const pb = w.initTensor(probe, [5]);

@@ -87,6 +87,9 @@ def test_js_gpt_on_gpu_matches_oracle():
         nxt = int(np.argmax(ref.forward(p, w, np.array(hist, np.int32))))
         assert nxt == out["generated"][i]
         hist.append(nxt)
+    # generate() in bursts: the tokens of a call per token
+    assert len(out["bursts"]["1"]) == 19
+    assert out["bursts"]["8"] == out["bursts"]["1"] and out["bursts"]["5"] == out["bursts"]["1"]
     # token selection on the device, through the addon (globals.js:47-74)
     want_id, want_ids, want_p = ref.sample_topk(np.array([0.5, 2.0, -1.0, 2.0, 1.5], np.float32), 3, 0.5, 0.6)
     assert out["select"]["id"] == want_id and out["select"]["topKIndices"] == [int(i) for i in want_ids]
