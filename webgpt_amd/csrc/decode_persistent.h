@@ -33,6 +33,9 @@ struct PhaseGeom {
 struct LayerParamOffsets {
   int bA, bC, bD, bE, ln1g, ln1b, ln2g, ln2b;
   int sA, sC, sD, sE;  // per-column scales of the int8 variant; for fp32 weights sA and sD hold the column sums of diag(gamma) W
+  // int8 variant, the two matrices behind a LayerNorm: gA, gD the column sums sum_k gamma_k q_kn of the quantised
+  // weights, fA, fD the biases with the LayerNorm's beta folded in, bias_n + scale_n / 127 sum_k beta_k q_kn (fold_ln_i8)
+  int gA, gD, fA, fD;
   int stride;
 };
 __host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
@@ -40,7 +43,8 @@ __host__ __device__ inline LayerParamOffsets layer_param_offsets(int d) {
   o.bA = 0; o.bC = 3 * d; o.bD = 4 * d; o.bE = 8 * d;
   o.ln1g = 9 * d; o.ln1b = 10 * d; o.ln2g = 11 * d; o.ln2b = 12 * d;
   o.sA = 13 * d; o.sC = 16 * d; o.sD = 17 * d; o.sE = 21 * d;
-  o.stride = 22 * d;
+  o.gA = 22 * d; o.gD = 25 * d; o.fA = 29 * d; o.fD = 32 * d;
+  o.stride = 36 * d;
   return o;
 }
 
@@ -53,7 +57,7 @@ struct PersistentArgs {
   // slabs + l*slab_stride; c_attn at 0, then attn c_proj, c_fc, mlp c_proj (item-lane units)
   const void* slabs;
   size_t slab_stride, slab_offC, slab_offD, slab_offE;
-  const float* lparams;  // [L][22d] small per-layer parameters (LayerParamOffsets)
+  const float* lparams;  // [L][36d] small per-layer parameters (LayerParamOffsets)
   const float* colparams;  // [L][PD_GRID][PD_COLP] biases and int8 scales / 127 per workgroup (build_colparams)
   const float *wte, *wpe, *lnf_g, *lnf_b;
   float* kv;  // [L][2][H][ctx][hs]
@@ -93,6 +97,11 @@ size_t slab_float4s(const PhaseGeom& g);
 // (the gamma of the LayerNorm in front of the matrix, or null) as diag(rowscale) W.
 hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const float* rowscale, float4* slab, hipStream_t s);
 // out[N] = bias + beta W: the beta of that LayerNorm folded into the bias; colsum[N] = column sums of diag(gamma) W.
+// The same for packed int8 weights (Wq[K, N/4] words, scale[N]; other/int8-gemm.js:36-43), whose gamma cannot be folded
+// into the quantised values: out_bias[n] = bias[n] + scale[n] / 127 sum_k beta[k] q[k][n], gsum[n] = sum_k gamma[k] q[k][n]
+// (both accumulated in double, rounded once).
+hipError_t fold_ln_i8(const int32_t* Wq, int ldwq, int K, int N, const float* scale, const float* gamma, const float* beta,
+                      const float* bias, float* out_bias, float* gsum, hipStream_t s);
 hipError_t fold_ln_bias(const float* W, int ldw, int K, int N, const float* gamma, const float* beta, const float* bias, float* out,
                         float* colsum, hipStream_t s);
 // Same for int8 words Wq[K, ldwq] (4 columns per word): one word per item lane.

@@ -459,6 +459,11 @@ __device__ __forceinline__ ColParams col_params(const float* colp, int ph, int c
 __device__ __forceinline__ float finish_ln(float dot, float mean, float rstd, const ColParams& cp) {
   return rstd * (dot - mean * cp.scale) + cp.bias;
 }
+// int8 items behind a LayerNorm (gemv_whole_ln8): gsum = sum_k gamma_k q_kn, scale the column scale / 127, and the
+// bias holds bias_n + scale sum_k beta_k q_kn.
+__device__ __forceinline__ float finish_ln8(float dot, float mean, float rstd, const ColParams& cp, float gsum) {
+  return (rstd * (dot - mean * gsum)) * cp.scale + cp.bias;
+}
 // Finished value of a column from its dot product: the int8 column scale, the bias last.
 template <bool I8>
 __device__ __forceinline__ float finish(float dot, const ColParams& cp) {
@@ -852,6 +857,51 @@ __device__ __forceinline__ float gemv_whole_ln(const WS& ws, const float* xs, in
   return val;
 }
 
+// The same behind a LayerNorm whose gamma is not in the weights (int8 items): the raw row times gamma (gam: LDS,
+// gamma followed by beta, so that a read beyond K meets finite values; the row is zero there) against the wave's
+// columns, the statistics of the raw row in the same reduction. sum_k ((x_k - mean) rstd gamma_k + beta_k) q_kn =
+// rstd (dot - mean G_n) + sum_k beta_k q_kn with dot = sum_k x_k gamma_k q_kn and G_n = sum_k gamma_k q_kn: the
+// caller finishes with G_n and a bias that holds the beta term (fold_ln_i8_kernel). `next` requests its items
+// between the items of this phase.
+template <class P, class WS, class R>
+__device__ __forceinline__ float gemv_whole_ln8(const WS& ws, const float* xs, const float* gam, int ncols, int wave, int lane,
+                                                float& mean, float& rstd, const R& next) {
+  static_assert(P::WHOLE, "phase is not laid out by whole columns");
+  const int l4 = opaque(lane) * 4;
+  float4 xr[P::S];
+  float red[2 + P::CW];
+  red[0] = 0.f;
+  red[1] = 0.f;
+#pragma unroll
+  for (int s2 = 0; s2 < P::S; ++s2) {
+    const float4 x = *reinterpret_cast<const float4*>(xs + s2 * SEG + l4);  // (zero beyond K)
+    const float4 g = *reinterpret_cast<const float4*>(gam + s2 * SEG + l4);
+    red[0] += (x.x + x.y) + (x.z + x.w);
+    red[1] += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+    xr[s2] = make_float4(x.x * g.x, x.y * g.y, x.z * g.z, x.w * g.w);
+  }
+  static_for<P::CW>([&](auto CC) {
+    constexpr int cc = decltype(CC)::value;
+    const bool valid = wave + cc * NW < (P::RAGGED ? ncols : P::CPW);
+    float acc = 0.f;
+    static_for<P::S>([&](auto SG) {
+      constexpr int seg = decltype(SG)::value;
+      if (valid) acc = item_sum<true>(acc, to_float4(ws.w[cc * P::S + seg]), xr[seg]);
+      next.template slot<cc * P::S + seg, P::CW * P::S>();
+      pin_requests<R>();
+    });
+    red[2 + cc] = acc;
+  });
+  wave_sum_n(red);
+  mean = red[0] * (1.0f / (float)P::K);
+  const float var = fmaxf(__builtin_fmaf(-mean, mean, red[1] * (1.0f / (float)P::K)), 0.f);
+  rstd = fast_rsqrt(var + 1e-5f);
+  float val = 0.f;
+#pragma unroll
+  for (int cc = 0; cc < P::CW; ++cc) val = lane == cc ? red[2 + cc] : val;
+  return val;
+}
+
 // Other phases: per (column, wave) partial sums go to part[col * NW + wave]. The item
 // code exists once per wave with every index a constant: a phase is short, and what
 // it costs is instruction count (a runtime-indexed single copy measured 5-15 %
@@ -1041,6 +1091,10 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
   // ... and the LayerNorm in front of c_attn and c_fc is an epilogue of the dot products (finish_ln; the fp32 d = 1600
   // shape spills six times as much with it)
   constexpr bool LNEPI = FOLD && LN_EPILOGUE && D <= 1280;
+  // int8 items: the same with gamma multiplied into the row instead of into the weights (gemv_whole_ln8). The column
+  // sums ride in the free slots of the projections' bias rows of colp (build_colparams_kernel).
+  constexpr bool LNEPI8 = I8 && LN_EPILOGUE;
+  static_assert(!LNEPI8 || (PC::CPW + PD::CPW <= LPW && PE::CPW + PA::CPW <= LPW), "no room for the column sums in colp");
   constexpr int XS0 = C::SD * SEG;                                  // floats of a D-long input row
   constexpr int XS1 = C::SH * SEG;                                  // floats of a HID-long input row
   constexpr int ATTP = C::ATTW > 2 * PD_TOPK * C::G ? C::ATTW : 2 * PD_TOPK * C::G;  // floats of the staged exchange words
@@ -1209,11 +1263,15 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         own_r = finC ? xs0[wg * PC::CPW + fc] : 0.f;
         const ColParams cp = col_params<true>(colp, PH, fc);  // second slot: int8 scale, or the column sum of a folded LayerNorm
         float dot, mean = 0.f, rstd = 1.f;
-        if constexpr (SPREAD) dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part, nextC);
+        if constexpr (SPREAD && LNEPI8) dot = gemv_whole_ln8<PA>(wX, xs0, lnp, ncA, wave, lane, mean, rstd, nextC);
+        else if constexpr (SPREAD) dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part, nextC);
         else if constexpr (LNEPI) dot = gemv_whole_ln<PA>(wX, xs0, ncA, wave, lane, mean, rstd);
         else dot = gemv_whole<PA, true, !FOLD>(wX, xs0, lnp, ncA, wave, lane, xs1, part);
         TRACE5(2);
-        if (finA) pubA[fc] = LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp);
+        if (finA) {
+          if constexpr (SPREAD && LNEPI8) pubA[fc] = finish_ln8(dot, mean, rstd, cp, colp[PH_FC2 * LPW + ((PE::CPW + fc) & (LPW - 1))]);
+          else pubA[fc] = LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp);
+        }
         __syncthreads();
         ++ep;
         if (tid < ncA) publish(a.bufQKV + wg * PA::CPW + tid, pubA[tid], ep);
@@ -1484,11 +1542,15 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         const ColParams cp = col_params<true>(colp, PH, fc);
         float dot, mean = 0.f, rstd = 1.f;
         const Leading<LoadE, SPN, SPD> leadE{nextE};
-        if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, leadE);
+        if constexpr (SPREAD && LNEPI8) dot = gemv_whole_ln8<PD>(wX, xs0, lnp, ncD, wave, lane, mean, rstd, leadE);
+        else if constexpr (SPREAD) dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part, leadE);
         else if constexpr (LNEPI) dot = gemv_whole_ln<PD>(wX, xs0, ncD, wave, lane, mean, rstd);
         else dot = gemv_whole<PD, true, !FOLD>(wX, xs0, lnp, ncD, wave, lane, xs1, part);
         TRACE5(2);
-        if (finD) pubD[fc] = gelu_ref(LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp));  // model.js:188
+        if (finD) {  // model.js:188
+          if constexpr (SPREAD && LNEPI8) pubD[fc] = gelu_ref(finish_ln8(dot, mean, rstd, cp, colp[PH_PROJ * LPW + ((PC::CPW + fc) & (LPW - 1))]));
+          else pubD[fc] = gelu_ref(LNEPI ? finish_ln(dot, mean, rstd, cp) : finish<I8>(dot, cp));
+        }
         __syncthreads();
         ++ep;
         if constexpr (!TRIPLE_H) {
@@ -1940,6 +2002,22 @@ __global__ void fold_ln_bias_kernel(const float* __restrict__ W, int ldw, int K,
   colsum[n] = (float)sum;
 }
 
+__global__ void fold_ln_i8_kernel(const int32_t* __restrict__ Wq, int ldwq, int K, int N, const float* __restrict__ scale,
+                                  const float* __restrict__ gamma, const float* __restrict__ beta, const float* __restrict__ bias,
+                                  float* __restrict__ out_bias, float* __restrict__ gsum) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  double bq = 0.0, gq = 0.0;
+  const int sh = 8 * (n & 3);
+  for (int k = 0; k < K; ++k) {
+    const int q = (int)(int8_t)(((unsigned)Wq[(size_t)k * ldwq + (n >> 2)] >> sh) & 0xffu);
+    bq += (double)beta[k] * (double)q;
+    gq += (double)gamma[k] * (double)q;
+  }
+  out_bias[n] = (float)((double)bias[n] + (double)(scale[n] / 127.0f) * bq);
+  gsum[n] = (float)gq;
+}
+
 // int8: item (w, j = c*S + seg, lane) is one word holding rows k..k+3 (k = seg*256 + lane*4)
 // of column w*cpw + c, gathered from the reference packing [K, N/4] (4 consecutive
 // columns per word, other/int8-gemm.js:36-43).
@@ -1972,14 +2050,22 @@ __global__ void build_colparams_kernel(const float* __restrict__ lparams, int L,
   const int kind = t / (4 * LPW), ph = (t / LPW) & 3, c = t % LPW;
   const LayerParamOffsets po = layer_param_offsets(d);
   const PhaseGeom g = ph == PH_QKV ? gA : ph == PH_PROJ ? gC : ph == PH_FC ? gD : gE;
-  const int off = ph == PH_QKV ? (kind ? po.sA : po.bA) : ph == PH_PROJ ? (kind ? po.sC : po.bC)
-                : ph == PH_FC ? (kind ? po.sD : po.bD) : (kind ? po.sE : po.bE);
+  // (int8: the two matrices behind a LayerNorm take their biases with beta folded in)
+  const int off = ph == PH_QKV ? (kind ? po.sA : i8 ? po.fA : po.bA) : ph == PH_PROJ ? (kind ? po.sC : po.bC)
+                : ph == PH_FC ? (kind ? po.sD : i8 ? po.fD : po.bD) : (kind ? po.sE : po.bE);
   const int col = wg * g.cpw + c;
   float v = 0.f;
   // second slot: int8 column scales, or for fp32 the column sums of the two matrices behind a LayerNorm
   if (c < g.cpw && col < g.N && (kind == 0 || i8 || ph == PH_QKV || ph == PH_FC)) {
     v = lparams[(size_t)layer * po.stride + off + col];
     if (kind && i8) v = v / 127.0f;  // other/int8-gemm.js:126-132 divides by 127 before the column scale is applied
+  }
+  // int8: the column sums sum_k gamma_k q_kn of those two matrices ride in the bias rows of the two projections, behind
+  // their (few) columns: c_fc's in attn c_proj's row, c_attn's in mlp c_proj's (col_gsum)
+  if (i8 && kind == 0 && (ph == PH_PROJ || ph == PH_FC2) && c >= g.cpw) {
+    const PhaseGeom gg = ph == PH_PROJ ? gD : gA;
+    const int c2 = c - g.cpw, col2 = wg * gg.cpw + c2;
+    if (c2 < gg.cpw && col2 < gg.N) v = lparams[(size_t)layer * po.stride + (ph == PH_PROJ ? po.gD : po.gA) + col2];
   }
   out[idx] = v;
 }
@@ -2038,6 +2124,12 @@ size_t slab_float4s(const PhaseGeom& g) { return (size_t)PD_GRID * g.cpw * g.S *
 hipError_t build_slab(const float* W, int ldw, int K, const PhaseGeom& g, const float* rowscale, float4* slab, hipStream_t s) {
   const size_t total = slab_float4s(g);
   build_slab_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(W, ldw, K, g.N, g.cpw, g.S, total, rowscale, slab);
+  return hipGetLastError();
+}
+
+hipError_t fold_ln_i8(const int32_t* Wq, int ldwq, int K, int N, const float* scale, const float* gamma, const float* beta,
+                      const float* bias, float* out_bias, float* gsum, hipStream_t s) {
+  fold_ln_i8_kernel<<<(unsigned)((N + 127) / 128), 128, 0, s>>>(Wq, ldwq, K, N, scale, gamma, beta, bias, out_bias, gsum);
   return hipGetLastError();
 }
 

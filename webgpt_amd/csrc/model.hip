@@ -348,6 +348,10 @@ static int setup_persistent(Model* m) {
     if (!i8) {
       LAUNCH(fold_ln_bias(l.attn.w, 3 * d, d, 3 * d, l.ln1_g, l.ln1_b, l.attn_b, lp + po.bA, lp + po.sA, rt().stream));
       LAUNCH(fold_ln_bias(l.fc.w, hid, d, hid, l.ln2_g, l.ln2_b, l.fc_b, lp + po.bD, lp + po.sD, rt().stream));
+    } else {
+      // (the plain biases stay where they are: the one-launch-per-block path applies the LayerNorm itself)
+      LAUNCH(fold_ln_i8(l.attn.q, 3 * d / 4, d, 3 * d, l.attn.s, l.ln1_g, l.ln1_b, l.attn_b, lp + po.fA, lp + po.gA, rt().stream));
+      LAUNCH(fold_ln_i8(l.fc.q, hid / 4, d, hid, l.fc.s, l.ln2_g, l.ln2_b, l.fc_b, lp + po.fD, lp + po.gD, rt().stream));
     }
   }
   a.slabs = slabs;
