@@ -649,23 +649,25 @@ __device__ __forceinline__ void pin_requests() {
 // LayerNorm parameters travel global memory -> registers (requested with the weights
 // of the phase) -> LDS (deposited next to the polled input row, before the barrier
 // that follows the poll): gamma at lnp[0, D), beta at lnp[D, 2D).
-template <int D, int NLN>
+// GAMMA_ONLY: a LayerNorm that is taken as an epilogue of int8 items needs no beta (it is in the folded bias).
+template <int D, bool GAMMA_ONLY = false, int NLN>
 __device__ __forceinline__ void request_ln(float4 (&r)[NLN], const float* __restrict__ gamma, const float* __restrict__ beta) {
   const int t = opaque(threadIdx.x);
 #pragma unroll
   for (int i = 0; i < NLN; ++i) {
     const int idx = t + i * NT;
+    if (GAMMA_ONLY && i * NT >= D / 4) continue;
     r[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (idx < D / 4) r[i] = reinterpret_cast<const float4*>(gamma)[idx];
-    else if (idx < D / 2) r[i] = reinterpret_cast<const float4*>(beta)[idx - D / 4];
+    else if (!GAMMA_ONLY && idx < D / 2) r[i] = reinterpret_cast<const float4*>(beta)[idx - D / 4];
   }
 }
-template <int D, int NLN>
+template <int D, bool GAMMA_ONLY = false, int NLN>
 __device__ __forceinline__ void deposit_ln(const float4 (&r)[NLN], float* lnp) {
   const int t = opaque(threadIdx.x);
 #pragma unroll
   for (int i = 0; i < NLN; ++i)
-    if (t + i * NT < D / 2) reinterpret_cast<float4*>(lnp)[t + i * NT] = r[i];
+    if (t + i * NT < (GAMMA_ONLY ? D / 4 : D / 2)) reinterpret_cast<float4*>(lnp)[t + i * NT] = r[i];
 }
 
 // The input row (LDS, zero padded up to S * SEG) as this lane's float4 of every
@@ -1251,7 +1253,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         [[maybe_unused]] constexpr int PH = PH_QKV;
         if (li > 0) {
           poll_words<D>(a.bufR2, ep, xs0, a.err, a.delay[0], a.spin_limit);
-          if (!FOLD) deposit_ln<D>(lnreg, lnp);
+          if (!FOLD) deposit_ln<D, LNEPI8>(lnreg, lnp);
           deposit_params();
           __syncthreads();
           if (sh.bail) return;
@@ -1439,7 +1441,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE(1 + li * 8 + PH);
         const LoadD nextD(wX, slab + a.slab_offD, ncD, wg, wave, lane);
         if (DUAL && !SPREAD) nextD.early();
-        if (DUAL && !FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
+        if (DUAL && !FOLD) request_ln<D, LNEPI8>(lnreg, lp + po.ln2g, lp + po.ln2b);
         // merge of the slices of each head (flash-decoding): element e of head h is
         // sum_s o_s[e] exp(m_s - M) / sum_s l_s exp(m_s - M), M = max_s m_s. The H * SPLIT normalised weights
         // exp(m_s - M) / sum are made once (thread h * SPLIT + s; `part` is idle between the attention and the
@@ -1523,7 +1525,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         TRACE5(4);
         if (!DUAL) {
           nextD.all();
-          if (!FOLD) request_ln<D>(lnreg, lp + po.ln2g, lp + po.ln2b);
+          if (!FOLD) request_ln<D, LNEPI8>(lnreg, lp + po.ln2g, lp + po.ln2b);
         } else if (!SPREAD) nextD.late();
         else leadD.rest();
         TRACE5(5);
@@ -1533,7 +1535,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       {
         [[maybe_unused]] constexpr int PH = PH_FC;
         poll_words<D>(a.bufR1, ep, xs0, a.err, a.delay[4], a.spin_limit);
-        if (!FOLD) deposit_ln<D>(lnreg, lnp);
+        if (!FOLD) deposit_ln<D, LNEPI8>(lnreg, lnp);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);
@@ -1579,7 +1581,7 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
         auto request_small = [&]() {
           if (li + 1 < a.L) {
             request_params(li + 1);
-            if (!FOLD) request_ln<D>(lnreg, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
+            if (!FOLD) request_ln<D, LNEPI8>(lnreg, lp + po.stride + po.ln1g, lp + po.stride + po.ln1b);
           } else {
             if (!FOLD) request_ln<D>(lnreg, a.lnf_g, a.lnf_b);
             if (step + 1 < a.nsteps) request_params(0);
