@@ -74,6 +74,9 @@ struct PersistentArgs {
   // [2] attention outputs on the attention workgroups, [3] on the others,
   // [4] residual row into c_fc, [5] hidden row, [6] arg-max candidates
   int delay[7];
+  // the attention slices take longer the longer the context: delay[2] and delay[3] grow by att_slope[0] and
+  // att_slope[1] units per 1024 positions of the step's context
+  int att_slope[2];
   unsigned spin_limit;  // poll rounds after which a wait gives up and raises *err
   int short_keys;       // a launch whose last step attends to more positions runs the instantiation with PD_SPLIT_LONG slices (<= PD_SHORT_KEYS)
   // token selection: top_k == 1 is the arg-max; 2..PD_TOPK samples as GPT.generate does

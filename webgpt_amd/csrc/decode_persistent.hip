@@ -1434,8 +1434,9 @@ __global__ __launch_bounds__(NT) void decode_persistent_kernel(PersistentArgs a)
       // ======================= attention c_proj: merge slices, project, residual =======================
       {
         [[maybe_unused]] constexpr int PH = PH_PROJ;
-        if constexpr (TRIPLE_ATT) poll_triples<C::ATTW / 3, 0>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
-        else poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_role ? a.delay[2] : a.delay[3], a.spin_limit);
+        const int att_delay = att_role ? a.delay[2] + ((pos * a.att_slope[0]) >> 10) : a.delay[3] + ((pos * a.att_slope[1]) >> 10);
+        if constexpr (TRIPLE_ATT) poll_triples<C::ATTW / 3, 0>(a.bufATT, ep, attp, a.err, att_delay, a.spin_limit);
+        else poll_words<C::ATTW>(a.bufATT, ep, attp, a.err, att_delay, a.spin_limit);
         __syncthreads();
         wait_loads();
         TRACE(1 + li * 8 + PH);

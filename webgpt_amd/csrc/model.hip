@@ -393,17 +393,28 @@ static int setup_persistent(Model* m) {
     // curves are flat within a few percent around them and over context length);
     // wgpt_model_tune_poll_delays searches around them on the GPU at hand,
     // WEBGPT_AMD_POLL_DELAYS="a,b,c,d,e,f,g" overrides them for experiments
-    static const int tuned[5][7] = {{16, 4, 32, 80, 24, 28, 48},    // d <= 768
-                                    {36, 0, 32, 104, 40, 40, 4},    // d = 1024
-                                    {20, 0, 36, 128, 16, 16, 52},   // d = 1280
-                                    {12, 12, 28, 104, 20, 12, 44},  // d = 1600, int8
+    static const int tuned[5][7] = {{16, 4, 22, 78, 24, 28, 48},    // d <= 768
+                                    {36, 0, 26, 82, 40, 40, 4},     // d = 1024
+                                    {20, 0, 34, 100, 16, 16, 52},   // d = 1280
+                                    {8, 12, 22, 84, 20, 12, 44},    // d = 1600, int8
                                     {32, 0, 48, 96, 4, 20, 40}};    // d = 1600, fp32
-    const int* dflt = tuned[d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4];
+    // growth of [2] and [3] per 1024 positions of context (the best values at contexts of 100, 350, 650 and 900
+    // positions lie on a line: 117M 80, 88, 88, 104 for [3]; int8 88, 104, 128, 136)
+    static const int slopes[5][2] = {{11, 28}, {0, 46}, {9, 70}, {20, 61}, {0, 0}};
+    const int row = d <= 768 ? 0 : d == 1024 ? 1 : d == 1280 ? 2 : i8 ? 3 : 4;
+    const int* dflt = tuned[row];
     for (int i = 0; i < 7; ++i) a.delay[i] = dflt[i];
+    a.att_slope[0] = slopes[row][0];
+    a.att_slope[1] = slopes[row][1];
     if (const char* e = getenv("WEBGPT_AMD_POLL_DELAYS")) {
       int v[7];
       if (sscanf(e, "%d,%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6]) == 7)
         for (int i = 0; i < 7; ++i) a.delay[i] = v[i] < 0 ? 0 : (v[i] > 1024 ? 1024 : v[i]);
+    }
+    if (const char* e = getenv("WEBGPT_AMD_POLL_SLOPES")) {
+      int v[2];
+      if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2)
+        for (int i = 0; i < 2; ++i) a.att_slope[i] = v[i] < 0 ? 0 : (v[i] > 1024 ? 1024 : v[i]);
     }
   }
   // a wait that takes this many poll rounds (a quarter of a second) means a workgroup is not running;
