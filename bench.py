@@ -83,10 +83,10 @@ def cpu_baseline(cfg, tensors, prompt, budget_s=20.0):
 # on single-token launches of the persistent kernel: bytes, the contexts of the profiled launches, the profile that
 # holds the figures and the first 16 hex digits of the SHA-256 of the kernel's source file when it was profiled.
 MEASURED_TRAFFIC = {
-    "gpt2-117m": (515.8e6, (133, 164), "profiles/decode_persistent_gpt2-117m.md", "2043c8780dbb7d12"),
-    "gpt2-345m": (1557.9e6, (555, 586), "profiles/decode_persistent_other_configs.md", "2043c8780dbb7d12"),
-    "gpt2-774m": (3182.2e6, (107, 138), "profiles/decode_persistent_other_configs.md", "2043c8780dbb7d12"),
-    "gpt2-1.5b-int8": (2122.2e6, (171, 202), "profiles/decode_persistent_other_configs.md", "2043c8780dbb7d12"),
+    "gpt2-117m": (515.8e6, (133, 164), "profiles/decode_persistent_gpt2-117m.md", "7b7ce1999a5b27ff"),
+    "gpt2-345m": (1557.9e6, (555, 586), "profiles/decode_persistent_other_configs.md", "7b7ce1999a5b27ff"),
+    "gpt2-774m": (3178.0e6, (107, 138), "profiles/decode_persistent_other_configs.md", "7b7ce1999a5b27ff"),
+    "gpt2-1.5b-int8": (2116.9e6, (171, 202), "profiles/decode_persistent_other_configs.md", "7b7ce1999a5b27ff"),
 }
 KERNEL_SOURCE = os.path.join(ROOT, "webgpt_amd", "csrc", "decode_persistent.hip")
 
